@@ -29,6 +29,7 @@ class CacheStorage:
         max_slots: int,
         dtype: torch.dtype,
         device: torch.device,
+        embedding_state_need: StateNeed | None = None,
     ):
         self.page_size = page_size
         self.keys: list[torch.Tensor] = []
@@ -47,6 +48,8 @@ class CacheStorage:
             return torch.zeros((max_slots + 1, *need.shape), dtype=need.dtype, device=device)
 
         self.states: list = [make(need) for need in state_needs]
+        # what the embedding keeps per request (the token before, for one that reads pairs of tokens)
+        self.embedding_state = make(embedding_state_need)
         # slot `max_slots` belongs to no request (padding rows of a recorded step use it)
         self.last_token = torch.zeros((max_slots + 1,), dtype=torch.int32, device=device)
 
@@ -55,7 +58,7 @@ class CacheStorage:
         starts from the state a fresh engine would give it, whoever held the slot before."""
         if not slots:
             return
-        for item in self.states:
+        for item in [*self.states, self.embedding_state]:
             for t in (item if isinstance(item, list) else [item]):
                 if t is not None:
                     for s in slots:

@@ -13,7 +13,8 @@
 // A query at position p sees positions max(0, p - window + 1) .. p (window <= 0: all).
 // Keys have d elements a head and values dv (dv = d in most models).  `sink` (null, or one
 // 32-bit number a query head): exp(sink) is added once to the softmax's denominator; it has no
-// key and no value.
+// key and no value.  `score_bias` (null, or one 32-bit number a query head): the weights are no
+// softmax but sigmoid(score + score_bias[head]) for every key the query sees, not normalised.
 #include "common.h"
 
 #define AG_THREADS 256
@@ -25,7 +26,7 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
     const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_req,
     const int* __restrict__ positions, int nq, int nkv, int d, int dv, int P, int window, float scale,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, const float* __restrict__ score_bias) {
   extern __shared__ float smem[];
   const int t = blockIdx.x, g = blockIdx.y;
   const int group = nq / nkv;
@@ -92,6 +93,12 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
     // softmax bookkeeping: one wavefront per query head, one position per lane
     for (int gq = wave; gq < group; gq += AG_THREADS / TK_WAVE) {
       const float s = lane < CH ? Ss[gq * CH + lane] : -INFINITY;
+      if (score_bias) {  // sigmoid weights: nothing to rescale, no sum to keep
+        const float p = (s == -INFINITY) ? 0.f : 1.0f / (1.0f + expf(-(s + score_bias[g * group + gq])));
+        if (lane < CH) Ss[gq * CH + lane] = p;
+        if (lane == 0) st_a[gq] = 1.f;
+        continue;
+      }
       const float m_old = st_m[gq];
       const float m_new = fmaxf(m_old, wave_max(s));
       const float p = (s == -INFINITY) ? 0.f : expf(s - m_new);
@@ -124,8 +131,8 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
     const int i = tid + r * AG_THREADS;
     if (i < n_out) {
       const int gq = i / dv;
-      float a = acc[r], l = st_l[gq];
-      if (sink) {
+      float a = acc[r], l = score_bias ? 1.f : st_l[gq];
+      if (sink && !score_bias) {
         // the sink joins the softmax like one more score: the maximum may rise to it
         const float sk = sink[g * group + gq], m = st_m[gq], m_all = fmaxf(m, sk);
         const float keep = expf(m - m_all);
@@ -146,11 +153,12 @@ template <typename T, int CH>
 static void ag_launch(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                       const void* vcache, const int* block_table, int table_stride,
                       const int* token_req, const int* positions, int n_tokens, int nq, int nkv,
-                      int d, int dv, int P, int window, float scale, const float* sink, hipStream_t stream) {
+                      int d, int dv, int P, int window, float scale, const float* sink, const float* score_bias,
+                      hipStream_t stream) {
   hipLaunchKernelGGL((paged_attention_generic_kernel<T, CH>), dim3(n_tokens, nkv),
                      dim3(AG_THREADS), ag_smem_bytes(nq / nkv, d, dv, CH), stream, (const T*)q,
                      q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache,
-                     block_table, table_stride, token_req, positions, nq, nkv, d, dv, P, window, scale, sink);
+                     block_table, table_stride, token_req, positions, nq, nkv, d, dv, P, window, scale, sink, score_bias);
 }
 
 // Whether the kernel takes this group and head size at all (0 and the reason in tk_last_error
@@ -171,7 +179,7 @@ TK_API int tk_paged_attention_generic(int dt, const void* q, int q_stride, void*
                                           const int* block_table, int table_stride,
                                           const int* token_req, const int* positions, int n_tokens,
                                           int nq, int nkv, int d, int dv, int P, int window, float scale,
-                                          const float* sink, hipStream_t stream) {
+                                          const float* sink, const float* score_bias, hipStream_t stream) {
   TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && P > 0 && nq % nkv == 0,
              "paged_attention: bad sizes tokens=%d nq=%d nkv=%d d=%d dv=%d P=%d", n_tokens, nq, nkv, d, dv,
              P);
@@ -189,7 +197,7 @@ TK_API int tk_paged_attention_generic(int dt, const void* q, int q_stride, void*
              "paged_attention: head size %d with group %d does not fit the local memory", d, group);
 #define AG_CASE(T, CHV)                                                                         \
   ag_launch<T, CHV>(q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride,    \
-                    token_req, positions, n_tokens, nq, nkv, d, dv, P, window, scale, sink, stream)
+                    token_req, positions, n_tokens, nq, nkv, d, dv, P, window, scale, sink, score_bias, stream)
   if (dt == TK_F32) {
     if (ch == 64) AG_CASE(float, 64);
     else if (ch == 32) AG_CASE(float, 32);

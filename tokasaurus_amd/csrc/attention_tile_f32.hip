@@ -2,7 +2,9 @@
 // softmax weights and the weighted values are 32-bit products of 32-bit operands, whatever the
 // storage type of queries, keys and values.  For mixers that ask for exactly that: a sliding
 // window, key and value heads of different sizes, a scale of the model's choosing and a
-// learned sink per query head in the softmax's denominator.
+// learned sink per query head in the softmax's denominator; or, with `score_bias` (one number a
+// query head), no softmax at all: a visible key's weight is sigmoid(score + score_bias[head]), not
+// normalised over the keys (the sums of wavefronts and chunks are then added as they are).
 //
 // A wavefront owns a tile of 16 "columns": tt = 16 / gg neighbouring tokens of one request
 // times gg neighbouring query heads of one kv head (gg = 1 for prompt portions; up to 16 for
@@ -45,7 +47,8 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     const T* __restrict__ vcache, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
     const int* __restrict__ tile_row0, int nq, int nkv, int dk, int dv, int P, int window, float scale,
-    const float* __restrict__ sink, int gg, int chunk = 0, float* __restrict__ part = nullptr) {
+    const float* __restrict__ sink, const float* __restrict__ score_bias, int gg, int chunk = 0,
+    float* __restrict__ part = nullptr) {
   extern __shared__ float merge[];  // SPLIT: [waves][16] maxima, [waves][16] sums, [waves - 1][VT][4][64] weighted values
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
   const int group = nq / nkv;
@@ -89,7 +92,10 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   v4f o[VT];
 #pragma unroll
   for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's share of the column's sum
+  const bool sig = score_bias != nullptr;
+  const float pb = sig && live ? score_bias[head] : 0.f;
+  // (sigmoid weights have no maximum to follow: it stays 0, so every merge below multiplies by exp(0))
+  float m_run = sig ? 0.f : -INFINITY, l_run = 0.f;  // l_run: this lane's share of the column's sum
 
   // where this lane's pieces of a key and its values lie inside a page, for the page's first key: both offsets
   // grow linearly with the key's place in the page (8 elements a key, dv a key)
@@ -179,22 +185,28 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
         tmax = fmaxf(tmax, sc[i]);
       }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, TK_WAVE));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, TK_WAVE));
-    const float m_new = fmaxf(m_run, tmax);
     float p[4];
     float alpha = 1.f;
-    if (m_new == -INFINITY) {
+    if (sig) {
+      // 1 / (1 + exp(-(score + bias))); a masked score gives 1 / (1 + inf) = 0
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p[i] = 0.f;
+      for (int i = 0; i < 4; ++i) p[i] = 1.0f / (1.0f + exp2f(-(sc[i] + pb) * 1.44269504088896341f));
     } else {
-      // exp2 of the difference times log2(e): the hardware's own exponential (a masked score gives exp2(-inf) = 0)
-      alpha = exp2f((m_run - m_new) * 1.44269504088896341f);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, TK_WAVE));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, TK_WAVE));
+      const float m_new = fmaxf(m_run, tmax);
+      if (m_new == -INFINITY) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p[i] = exp2f((sc[i] - m_new) * 1.44269504088896341f);
+        for (int i = 0; i < 4; ++i) p[i] = 0.f;
+      } else {
+        // exp2 of the difference times log2(e): the hardware's own exponential (a masked score gives exp2(-inf) = 0)
+        alpha = exp2f((m_run - m_new) * 1.44269504088896341f);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[i] = exp2f((sc[i] - m_new) * 1.44269504088896341f);
+      }
+      m_run = m_new;
+      l_run = l_run * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
     }
-    m_run = m_new;
-    l_run = l_run * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
     // O^T += V^T P^T
 #pragma unroll
     for (int t = 0; t < VT; ++t) {
@@ -270,14 +282,14 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     return;
   }
   float keep = 1.f;
-  if (sink && live) {
+  if (sink && live && !sig) {
     // the sink joins the softmax like one more score: the maximum may rise to it
     const float sk = sink[head], m_all = fmaxf(m_run, sk);
     keep = (m_run == -INFINITY) ? 0.f : expf(m_run - m_all);
     l = l * keep + expf(sk - m_all);
   }
   if (!live) return;
-  const float inv = keep / l;
+  const float inv = sig ? 1.f : keep / l;
   T* dst = out + (size_t)tok * out_stride + (size_t)head * dv;
 #pragma unroll
   for (int t = 0; t < VT; ++t) {
@@ -294,7 +306,7 @@ template <typename T, int VT>
 __global__ __launch_bounds__(VT * TK_WAVE) void attention_tile_merge_kernel(
     const float* __restrict__ part, int chunks, T* __restrict__ out, int out_stride, const int* __restrict__ q_start,
     const int* __restrict__ tile_req, const int* __restrict__ tile_row0, int nq, int nkv, int dv,
-    const float* __restrict__ sink, int gg) {
+    const float* __restrict__ sink, int gg, int plain_sums) {
   const int lane = threadIdx.x & (TK_WAVE - 1), t = threadIdx.x / TK_WAVE;
   if (16 * t >= dv) return;
   const int group = nq / nkv, blocks_per_kv = group / gg;
@@ -324,13 +336,13 @@ __global__ __launch_bounds__(VT * TK_WAVE) void attention_tile_merge_kernel(
     for (int i = 0; i < 4; ++i) o[i] = fmaf(oz[i], f, o[i]);
   }
   float keep = 1.f;
-  if (sink && live) {
+  if (sink && live && !plain_sums) {
     const float sk = sink[head], m2 = fmaxf(m_all, sk);
     keep = (m_all == -INFINITY) ? 0.f : expf(m_all - m2);
     l = l * keep + expf(sk - m2);
   }
   if (!live) return;
-  const float inv = keep / l;
+  const float inv = plain_sums ? 1.f : keep / l;  // (sigmoid weights: every chunk's maximum is 0 and its sums count as they are)
   T* dst = out + (size_t)tok * out_stride + (size_t)head * dv;
 #pragma unroll
   for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[i] * inv);
@@ -353,28 +365,28 @@ template <typename T, int KM, int VT>
 static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, int q_stride, void* out, int out_stride,
                       const void* kcache, const void* vcache, const int* block_table, int table_stride,
                       const int* q_start, const int* kv_len, const int* tile_req, const int* tile_row0, int nq,
-                      int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg, int chunk,
-                      float* part) {
+                      int nkv, int dk, int dv, int P, int window, float scale, const float* sink, const float* score_bias,
+                      int gg, int chunk, float* part) {
   if (split && chunk > 0) {
     constexpr int NW = VT <= 4 ? 8 : 4;
     const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW, true>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
-                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg,
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg,
                        chunk, part);
     hipLaunchKernelGGL((attention_tile_merge_kernel<T, VT>), dim3(grid.x, grid.y), dim3(VT * TK_WAVE), 0, stream, part, (int)grid.z,
-                       (T*)out, out_stride, q_start, tile_req, tile_row0, nq, nkv, dv, sink, gg);
+                       (T*)out, out_stride, q_start, tile_req, tile_row0, nq, nkv, dv, sink, gg, score_bias ? 1 : 0);
   } else if (split) {
     // eight wavefronts a tile where their sums fit the local memory, else four
     constexpr int NW = VT <= 4 ? 8 : 4;
     const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
-                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg);
   } else {
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, false, AT_WAVES>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
-                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg);
   }
 }
 
@@ -383,8 +395,9 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
 TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                                  const void* vcache, const int* block_table, int table_stride, const int* q_start,
                                  const int* kv_len, const int* tile_req, const int* tile_row0, int n_tiles, int nq,
-                                 int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg,
-                                 int split, int chunk, int chunks, float* part, hipStream_t stream) {
+                                 int nkv, int dk, int dv, int P, int window, float scale, const float* sink,
+                                 const float* score_bias, int gg, int split, int chunk, int chunks, float* part,
+                                 hipStream_t stream) {
   TK_REQUIRE(tk_attention_tile_f32_fits(nq, nkv, dk, dv, P), "attention_tile_f32: shape nq=%d nkv=%d dk=%d dv=%d P=%d not taken",
              nq, nkv, dk, dv, P);
   const int group = nq / nkv;
@@ -400,7 +413,7 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
   const dim3 grid(n_tiles, sp ? head_blocks : (head_blocks + AT_WAVES - 1) / AT_WAVES, parts ? chunks : 1);
   TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
 #define AT_ARGS grid, sp, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \
-                tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg, parts ? chunk : 0, part
+                tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, parts ? chunk : 0, part
 #define AT_VT(T, KMV)                                      \
   do {                                                     \
     if (vt <= 2) at_launch<T, KMV, 2>(AT_ARGS);            \

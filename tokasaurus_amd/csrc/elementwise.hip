@@ -257,6 +257,66 @@ TK_API int tk_swiglu(int dt, const void* gate_up, void* out, int rows, int inter
 }
 
 // --------------------------------------------------------------------------
+// A gated feed-forward's activation with clamps, on a fused [rows, 2*inter] product laid out
+// [gate | up]:  g = min(gate, limit), u = clamp(up, -limit, limit),
+//               out = g * sigmoid(alpha * g) * (u + 1), computed in 32-bit and rounded once.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, float limit, float alpha) {
+  const T* g = gu + (size_t)blockIdx.y * 2 * inter;
+  const T* u = g + inter;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < inter) {
+    const float gv = fminf(to_f32<T>(g[i]), limit);
+    const float uv = fminf(fmaxf(to_f32<T>(u[i]), -limit), limit);
+    out[(size_t)blockIdx.y * inter + i] = from_f32<T>(gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void clamped_glu_packed_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, float limit,
+                                                                 float alpha) {
+  constexpr int N = Pack<T>::N;
+  const int piece = blockIdx.x * blockDim.x + threadIdx.x;
+  if (piece >= inter / N) return;
+  const T* g = gu + (size_t)blockIdx.y * 2 * inter + (size_t)piece * N;
+  Pack<T> gv, uv, o;
+  gv.load(g);
+  uv.load(g + inter);
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float x = fminf(to_f32<T>(gv.v[j]), limit);
+    const float y = fminf(fmaxf(to_f32<T>(uv.v[j]), -limit), limit);
+    o.v[j] = from_f32<T>(x / (1.0f + expf(-alpha * x)) * (y + 1.0f));
+  }
+  o.store(out + (size_t)blockIdx.y * inter + (size_t)piece * N);
+}
+
+template <typename T>
+static void launch_clamped_glu(const void* gate_up, void* out, int rows, int inter, float limit, float alpha, hipStream_t stream) {
+  constexpr int N = Pack<T>::N;
+  if (inter % N == 0 && aligned16(gate_up) && aligned16(out))
+    hipLaunchKernelGGL(clamped_glu_packed_kernel<T>, dim3((inter / N + 255) / 256, rows), dim3(256), 0, stream,
+                       (const T*)gate_up, (T*)out, inter, limit, alpha);
+  else
+    hipLaunchKernelGGL(clamped_glu_kernel<T>, dim3((inter + 255) / 256, rows), dim3(256), 0, stream,
+                       (const T*)gate_up, (T*)out, inter, limit, alpha);
+}
+
+TK_API int tk_clamped_glu(int dt, const void* gate_up, void* out, int rows, int inter, float limit, float alpha,
+                          hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && inter > 0 && limit > 0.f, "clamped_glu: bad sizes %d %d or limit", rows, inter);
+  TK_REQUIRE(rows < 65536, "clamped_glu: %d rows are too many for one call", rows);
+  if (rows == 0) return 0;
+  if (dt == TK_F32)
+    launch_clamped_glu<float>(gate_up, out, rows, inter, limit, alpha, stream);
+  else
+    launch_clamped_glu<bf16_t>(gate_up, out, rows, inter, limit, alpha, stream);
+  TK_CHECK_LAUNCH("clamped_glu");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
 // gather_rows: out[i, :] = src[idx[i], :]   (src rows `src_stride` elements apart)
 // --------------------------------------------------------------------------
 template <typename T>

@@ -39,6 +39,83 @@ TK_API int tk_embed_scaled(int dt, const int* ids, const int* last_token, const 
 }
 
 // --------------------------------------------------------------------------
+// out[t, :] = float(table[id_t, :]) * scale + float(pairs[row_t, :]) where row_t is a hash of the
+// token before and the token itself, (prev * mul_prev + id * mul_cur) mod buckets, and row `buckets`
+// (the table's last) for a request's first token.  The token before is the one in front of it in this
+// step, or, for the first token that a request brings in a step, the one kept in the request's slot
+// (`prev_token`), where the workgroup of that first token then leaves the last token that the request
+// brings in this step (it alone reads and writes the slot's entry).  `cast` (null or T rows): the
+// same rows rounded once to the storage type.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_bigram_kernel(const int* __restrict__ ids, const int* __restrict__ last_token, const int* __restrict__ positions,
+                                    const int* __restrict__ token_req, const int* __restrict__ q_start, const int* __restrict__ slots,
+                                    int* __restrict__ prev_token, const T* __restrict__ table, const T* __restrict__ pairs,
+                                    float* __restrict__ out, T* __restrict__ cast, int hidden, int vocab, float scale,
+                                    int buckets, int mul_prev, int mul_cur) {
+  const int t = blockIdx.x;
+  const int r = token_req[t];
+  const int first = q_start[r], last = q_start[r + 1] - 1;
+  auto token_at = [&](int i) {
+    int id = ids[i];
+    if (id < 0) id = last_token[-id - 1];
+    return min(max(id, 0), vocab - 1);
+  };
+  const int id = token_at(t);
+  int row = buckets;
+  if (positions[t] > 0) {
+    const int prev = t > first ? token_at(t - 1) : prev_token[slots[r]];
+    row = (int)(((long long)prev * mul_prev + (long long)id * mul_cur) % buckets);
+  }
+  if (t == first && threadIdx.x == 0) prev_token[slots[r]] = token_at(last);
+  const T* src = table + (size_t)id * hidden;
+  const T* add = pairs + (size_t)row * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = fmaf(to_f32<T>(src[i]), scale, to_f32<T>(add[i]));
+    out[(size_t)t * hidden + i] = v;
+    if (cast) cast[(size_t)t * hidden + i] = from_f32<T>(v);
+  }
+}
+
+TK_API int tk_embed_bigram(int dt, const int* ids, const int* last_token, const int* positions, const int* token_req,
+                           const int* q_start, const int* slots, int* prev_token, const void* table, const void* pairs,
+                           float* out, void* cast, int n_tokens, int hidden, int vocab, float scale, int buckets,
+                           int mul_prev, int mul_cur, hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0 && buckets > 0, "embed_bigram: bad sizes %d %d %d %d", n_tokens, hidden, vocab, buckets);
+  TK_REQUIRE(ids && positions && token_req && q_start && slots && prev_token && table && pairs && out, "embed_bigram: a pointer is missing");
+  if (n_tokens == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(embed_bigram_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, ids, last_token, positions, token_req, q_start,
+                       slots, prev_token, (const float*)table, (const float*)pairs, out, (float*)nullptr, hidden, vocab, scale, buckets,
+                       mul_prev, mul_cur);
+  else
+    hipLaunchKernelGGL(embed_bigram_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, ids, last_token, positions, token_req, q_start,
+                       slots, prev_token, (const bf16_t*)table, (const bf16_t*)pairs, out, (bf16_t*)cast, hidden, vocab, scale, buckets,
+                       mul_prev, mul_cur);
+  TK_CHECK_LAUNCH("embed_bigram");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// out = T(x): a 32-bit stream rounded once to the storage type that a product reads.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void cast_rows_kernel(const float* __restrict__ x, T* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<T>(x[i]);
+}
+
+TK_API int tk_cast_rows(int dt, const float* x, void* out, size_t n, hipStream_t stream) {
+  TK_REQUIRE(dt == TK_BF16 && x && out, "cast_rows: 32-bit rows to bfloat16 rows");
+  if (n == 0) return 0;
+  const size_t blocks = (n + 255) / 256;
+  TK_REQUIRE(blocks < (1u << 31), "cast_rows: too many values");
+  hipLaunchKernelGGL(cast_rows_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, x, (bf16_t*)out, n);
+  TK_CHECK_LAUNCH("cast_rows");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
 // One row a workgroup.  Reads x (32-bit) and the branches a, b (32-bit, either may be null),
 // writes x_out = x + mult * (a + b) (32-bit; may be x itself; null when there is no branch and
 // the stream stays as it is) and, for each of up to two norms, the row
@@ -164,7 +241,8 @@ TK_API int tk_residual_norm(int dt, const float* x, const float* a, const float*
 // behind every sublayer), one row a workgroup:
 //     x_out = x + a / sqrt(mean(a^2) + eps_b) * wb
 // and, when w is given, the row of the norm that reads the new stream,
-//     h = x_out / sqrt(mean(x_out^2) + eps) * w     rounded once to T.
+//     h = x_out / sqrt(mean(x_out^2) + eps) * w     rounded once to T;
+// with h and no w, h is x_out itself rounded once to T (for sublayers that read the stream unnormed).
 // x, a, wb, w are 32-bit.  x_out may be x itself.  The row is held in registers between the
 // passes when the width allows (multiples of 4 up to 4 * 256 * RN_QUADS), else read back.
 // --------------------------------------------------------------------------
@@ -186,7 +264,11 @@ __global__ __launch_bounds__(256) void post_norm_residual_kernel(
     x_out[row + i] = v;
     ss = fmaf(v, v, ss);
   }
-  if (!w) return;
+  if (!h) return;
+  if (!w) {  // the new stream itself, rounded once
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) h[row + i] = from_f32<T>(x_out[row + i]);
+    return;
+  }
   const float rstd = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
   for (int i = threadIdx.x; i < hidden; i += blockDim.x)  // a thread reads back what it wrote
     h[row + i] = from_f32<T>(x_out[row + i] * rstd * w[i]);
@@ -225,13 +307,13 @@ __global__ __launch_bounds__(256) void post_norm_residual_vec_kernel(
       ss = fmaf(v[j].z, v[j].z, ss); ss = fmaf(v[j].w, v[j].w, ss);
     }
   }
-  if (!w) return;
-  const float rstd = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
+  if (!h) return;
+  const float rstd = w ? 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps) : 1.f;
 #pragma unroll
   for (int j = 0; j < RN_QUADS; ++j) {
     const int i = threadIdx.x + j * 256;
     if (i < quads) {
-      const float4 g = ((const float4*)w)[i];
+      const float4 g = w ? ((const float4*)w)[i] : make_float4(1.f, 1.f, 1.f, 1.f);
       const float n[4] = {v[j].x * rstd * g.x, v[j].y * rstd * g.y, v[j].z * rstd * g.z, v[j].w * rstd * g.w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) h[row + 4 * i + e] = from_f32<T>(n[e]);
@@ -243,6 +325,7 @@ TK_API int tk_post_norm_residual(int dt, const float* x, const float* a, const f
                                  const float* w, float eps, void* h, int rows, int hidden, hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && hidden > 0, "post_norm_residual: bad sizes %d %d", rows, hidden);
   TK_REQUIRE(x && a && wb && x_out && (!w || h), "post_norm_residual: a pointer is missing");
+  TK_REQUIRE(w || !h || dt != TK_F32, "post_norm_residual: 32-bit rows of the stream itself are the stream");
   if (rows == 0) return 0;
   const uintptr_t all = (uintptr_t)x | (uintptr_t)a | (uintptr_t)wb | (uintptr_t)x_out | (uintptr_t)w;
   const bool vec = hidden % 4 == 0 && hidden <= 4 * 256 * RN_QUADS && (all & 15) == 0;
@@ -287,6 +370,21 @@ TK_API int tk_concat_cast(int dt, const float* x, const float* y, void* out, int
 __global__ void softcap_kernel(float* __restrict__ v, size_t n, float cap) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) v[i] = cap * tanhf(v[i] / cap);
+}
+
+// logits <- logits * scale, in place, 32-bit.
+__global__ void scale_values_kernel(float* __restrict__ v, size_t n, float scale) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) v[i] = v[i] * scale;
+}
+
+TK_API int tk_scale_values(float* v, size_t n, float scale, hipStream_t stream) {
+  if (n == 0) return 0;
+  const size_t blocks = (n + 255) / 256;
+  TK_REQUIRE(v && blocks < (1u << 31), "scale_values: bad arguments");
+  hipLaunchKernelGGL(scale_values_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, v, n, scale);
+  TK_CHECK_LAUNCH("scale_values");
+  return 0;
 }
 
 TK_API int tk_softcap(float* v, size_t n, float cap, hipStream_t stream) {

@@ -226,7 +226,7 @@ class RecordedDecodeStep:
             token_ids=view("token_ids"), positions=view("positions"), token_req=view("token_req"),
             q_start=view("q_start"), kv_len=view("kv_len"), slots=view("slots"),
             host_q_start=list(range(B + 1)), host_kv_len=[kv_bound] * B, host_slots=[self.null_slot] * B,
-            last_token=storage.last_token, max_q_len=1, max_kv_len=kv_bound,
+            last_token=storage.last_token, embedding_state=storage.embedding_state, max_q_len=1, max_kv_len=kv_bound,
         )
         self.ctx.extras["static"] = True  # parts keep what they plan: the step is replayed
         self.ctx.extras["kv_bound"] = kv_bound
@@ -420,6 +420,7 @@ class ModelRunner:
             max_slots,
             model.dtype,
             model.device,
+            embedding_state_need=model.embedding_state_need(),
         )
 
     # ---- construction from a model folder
@@ -615,6 +616,7 @@ class ModelRunner:
             hb = layout(planned, self.model.spec.vocab_size, len(self.groups), self.manager.slot_tables)
             ctx, want_rows, tables = to_device(hb, self.model.dtype, self.model.device, self.storage.last_token)
             ctx.extras["kv_bound"] = self.kv_bound(ctx.max_kv_len)
+            ctx.embedding_state = self.storage.embedding_state
             every_row = hb.want_rows == list(range(ctx.num_tokens))
             logits = self.model.forward(ctx, self.cache_views(tables), self.storage.states, None if every_row else want_rows)
             out = StepOutput(logits)

@@ -35,13 +35,19 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_head_rmsnorm": [c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P],
         "tk_paged_attention_generic": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P]
         + [c_int] * 7
-        + [c_float, _P, _P],
+        + [c_float, _P, _P, _P],
         "tk_paged_attention_generic_fits": [c_int, c_int, c_int, c_int],
         "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
         "tk_embed_scaled": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
         "tk_residual_norm": [c_int, _P, _P, _P, c_float, _P, _P, _P, c_float, c_float, _P, _P, c_int, c_int, _P],
         "tk_softcap": [_P, c_size_t, c_float, _P],
-        "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 11 + [_P],
+        "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 13 + [_P, c_int, c_float, _P],
+        "tk_unrotate_gate": [c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P],
+        "tk_min_gru": [c_int, _P, c_int, _P, c_size_t, _P, _P, _P, c_int, c_int, c_int, _P],
+        "tk_embed_bigram": [c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P],
+        "tk_cast_rows": [c_int, _P, _P, c_size_t, _P],
+        "tk_scale_values": [_P, c_size_t, c_float, _P],
+        "tk_clamped_glu": [c_int, _P, _P, c_int, c_int, c_float, c_float, _P],
         "tk_gather_keys": [c_int, _P, _P, c_int, _P, _P, _P] + [c_int] * 5 + [_P],
         "tk_post_norm_residual": [c_int, _P, _P, _P, c_float, _P, _P, c_float, _P, c_int, c_int, _P],
         "tk_concat_cast": [c_int, _P, _P, _P, c_int, c_int, _P],
@@ -51,7 +57,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_head_linear": [c_int, _P, c_int, _P, _P, c_int, c_int] + [c_int] * 4 + [_P],
         "tk_squared_relu": [c_int, _P, c_size_t, _P],
         "tk_attention_tile_f32": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P] + [c_int] * 7
-        + [c_float, _P, c_int, c_int, c_int, c_int, _P, _P],
+        + [c_float, _P, _P, c_int, c_int, c_int, c_int, _P, _P],
         "tk_attention_tile_part_words": [c_int],
         "tk_attention_tile_f32_fits": [c_int] * 5,
         "tk_delta_prepare": [c_int, _P, c_int, c_int, _P, c_int, _P, c_int, _P, _P, _P, c_size_t, c_size_t, _P, _P, _P, _P]

@@ -355,14 +355,17 @@ def paged_attention_generic(
     scale: float | None = None,
     value_dim: int | None = None,
     sink: torch.Tensor | None = None,
+    score_bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Attention of every token over its request's pages (see rope_append for
     the page layout).  ``q`` is 2-d, its first nq*d columns are the query heads.
     ``value_dim``: the size of a value head (a key head's by default); the result is
     [tokens, nq * value_dim].  ``sink`` (32-bit, one number a query head): exp(sink) joins the
-    softmax's denominator once, with no key and no value."""
-    _gpu(q, kcache, vcache, block_table, token_req, positions, sink)
+    softmax's denominator once, with no key and no value.  ``score_bias`` (32-bit, one number a
+    query head): no softmax; a visible key's weight is sigmoid(score + score_bias[head]), not normalised."""
+    _gpu(q, kcache, vcache, block_table, token_req, positions, sink, score_bias)
     vd = head_dim if value_dim is None else int(value_dim)
+    _f32_vector(score_bias, nq, "attention: the scores' biases")
     _need(sink is None or (sink.shape == (nq,) and sink.dtype == torch.float32 and sink.is_contiguous()),
           f"attention: the sinks must be contiguous float32 [{nq}]")
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * head_dim,
@@ -397,6 +400,7 @@ def paged_attention_generic(
         int(window),
         float(scale if scale is not None else 1.0 / math.sqrt(head_dim)),
         sink.data_ptr() if sink is not None else None,
+        score_bias.data_ptr() if score_bias is not None else None,
         _stream(),
     )
     return out
@@ -1158,6 +1162,105 @@ def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
     return logits
 
 
+def scale_(logits: torch.Tensor, scale: float) -> torch.Tensor:
+    """logits <- logits * scale, in place (contiguous float32)."""
+    _gpu(logits)
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "scale: logits must be contiguous float32")
+    call("tk_scale_values", logits.data_ptr(), logits.numel(), float(scale), _stream())
+    return logits
+
+
+def cast_rows(x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """A 32-bit stream rounded once to ``out_dtype`` (the stream itself when that is 32-bit)."""
+    if out_dtype == torch.float32:
+        return x
+    _gpu(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "cast_rows: contiguous float32 rows")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    call("tk_cast_rows", dtype_code(out_dtype), x.data_ptr(), out.data_ptr(), x.numel(), _stream())
+    return out
+
+
+def embed_bigram(ctx_ids: torch.Tensor, last_token: torch.Tensor | None, positions: torch.Tensor, token_req: torch.Tensor,
+                 q_start: torch.Tensor, slots: torch.Tensor, prev_token: torch.Tensor, table: torch.Tensor, pairs: torch.Tensor,
+                 scale: float, mul_prev: int, mul_cur: int, want_cast: bool = True) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """The first rows of a 32-bit stream: ``table[id] * scale + pairs[(prev * mul_prev + id * mul_cur) mod buckets]``
+    where ``pairs`` has buckets + 1 rows and a request's first token (position 0) takes the last.  ``prev`` is
+    the token in front in this step or, for a request's first token of the step, ``prev_token[slot]``, which
+    is then set to the request's last token of this step.  Also returns the rows rounded once to the
+    table's type (None when that is 32-bit or ``want_cast`` is off)."""
+    _gpu(ctx_ids, last_token, positions, token_req, q_start, slots, prev_token, table, pairs)
+    for t, name in ((ctx_ids, "ids"), (positions, "positions"), (token_req, "token_req"), (q_start, "q_start"), (slots, "slots"),
+                    (prev_token, "prev_token")):
+        _i32(t, name)
+    if last_token is not None:
+        _i32(last_token, "last_token")
+    _need(table.dim() == 2 and table.is_contiguous() and pairs.dim() == 2 and pairs.is_contiguous() and pairs.dtype == table.dtype
+          and pairs.shape[1] == table.shape[1] and pairs.shape[0] >= 2, "embed_bigram: tables [V, H] and [buckets + 1, H] of one type")
+    n = ctx_ids.numel()
+    vocab, hidden = table.shape
+    _need(positions.numel() == n and token_req.numel() == n, "embed_bigram: one position and one request a token")
+    out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+    cast = torch.empty((n, hidden), dtype=table.dtype, device=table.device) if (want_cast and table.dtype != torch.float32) else None
+    call("tk_embed_bigram", dtype_code(table.dtype), ctx_ids.data_ptr(), last_token.data_ptr() if last_token is not None else None,
+         positions.data_ptr(), token_req.data_ptr(), q_start.data_ptr(), slots.data_ptr(), prev_token.data_ptr(), table.data_ptr(),
+         pairs.data_ptr(), out.data_ptr(), cast.data_ptr() if cast is not None else None, n, hidden, vocab, float(scale),
+         pairs.shape[0] - 1, int(mul_prev), int(mul_cur), _stream())
+    return out, cast
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """[rows, 2I] laid out [gate | up] -> g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit) and
+    u = clamp(up, -limit, limit), [rows, I]; 32-bit arithmetic, one rounding."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "clamped_glu input must be contiguous [rows, 2I]")
+    rows, two_i = gate_up.shape
+    out = torch.empty((rows, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    call("tk_clamped_glu", dtype_code(gate_up.dtype), gate_up.data_ptr(), out.data_ptr(), rows, two_i // 2, float(limit), float(alpha),
+         _stream())
+    return out
+
+
+def min_gru(proj: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, slots: torch.Tensor, width: int, longest: int,
+            out_dtype: torch.dtype) -> torch.Tensor:
+    """The gated recurrence ``S <- (1 - z) S + z cand`` per channel over every request's tokens of this
+    step, from and to the request's slot of ``state`` [slots, width] (32-bit): ``proj`` holds the 32-bit
+    sums [a | u | g] ([tokens, 3 width]; z = sigmoid(a), cand = u + 1/2 for u >= 0 and sigmoid(u) below);
+    returns S_t * silu(g) rounded once to ``out_dtype``.  ``longest``: the most tokens a request brings."""
+    _gpu(proj, state, q_start, slots)
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1 and proj.shape[1] >= 3 * width,
+          "min_gru: 32-bit rows [a | u | g]")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.stride(1) == 1 and state.shape[1] >= width,
+          "min_gru: the state is 32-bit [slots, width]")
+    _i32(q_start, "q_start")
+    _i32(slots, "slots")
+    _need(q_start.numel() == slots.numel() + 1, "min_gru: one slot a request")
+    out = torch.empty((proj.shape[0], width), dtype=out_dtype, device=proj.device)
+    call("tk_min_gru", dtype_code(out_dtype), proj.data_ptr(), proj.stride(0), state.data_ptr(), state.stride(0), q_start.data_ptr(),
+         slots.data_ptr(), out.data_ptr(), slots.numel(), int(width), int(longest), _stream())
+    return out
+
+
+def unrotate_gate_(o: torch.Tensor, positions: torch.Tensor | None, value_freq: torch.Tensor | None, pair_halves: bool,
+                   gate: torch.Tensor | None, nq: int, value_dim: int) -> torch.Tensor:
+    """In place on the heads' results [tokens, nq * value_dim]: pair m of every head turned by
+    -position * value_freq[m] (pairs as in ``qk_prepare``'s ``value_freq``), then head h times
+    sigmoid(gate[token, h]); ``gate`` is a 2-d view (rows may be strided) of the rows' type."""
+    _gpu(o, positions, value_freq, gate)
+    _need(o.dim() == 2 and o.stride(1) == 1 and o.shape[1] >= nq * value_dim, "unrotate_gate: rows of nq * dv")
+    if value_freq is not None:
+        _i32(positions, "positions")
+        _need(positions.numel() == o.shape[0], "unrotate_gate: one position a token")
+        _f32_vector(value_freq, value_dim // 2, "unrotate_gate: the values' frequencies")
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.stride(1) == 1 and gate.shape == (o.shape[0], nq) and gate.dtype == o.dtype,
+              "unrotate_gate: one gate a token and head, of the rows' type")
+    call("tk_unrotate_gate", dtype_code(o.dtype), o.data_ptr(), o.stride(0), positions.data_ptr() if value_freq is not None else None,
+         value_freq.data_ptr() if value_freq is not None else None, 1 if pair_halves else 0,
+         gate.data_ptr() if gate is not None else None, gate.stride(0) if gate is not None else 0, o.shape[0], nq, value_dim, _stream())
+    return o
+
+
 # --------------------------------------------------------------------------
 # attention with norms over the whole projection and a rotation of neighbouring elements
 # --------------------------------------------------------------------------
@@ -1182,6 +1285,11 @@ def qk_prepare(
     query_dim: int | None = None,
     pair_halves: bool = False,
     values_are_keys: bool = False,
+    per_head: bool = False,
+    key_skip: int = 0,
+    value_freq: torch.Tensor | None = None,
+    value_pair_halves: bool = False,
+    rotation_scale: float = 1.0,
 ) -> None:
     """In place on the rows [q: nq*dq | k: nkv*dk | v: nkv*dv] (only q when not ``write_cache``):
     the RMS norm of the whole query row and of the whole key row (32-bit weights of those sizes,
@@ -1190,19 +1298,27 @@ def qk_prepare(
     ``query_dim``: the size dq of a query head where it is not a key head's.  ``pair_halves``:
     the rotation pairs element i with element i + len(freq) instead of neighbours.
     ``values_are_keys``: the rows hold no values; a token's values are its keys as they are
-    before the rotation (after the norm, when there is one)."""
-    _gpu(qkv, positions, token_req, block_table, q_weight, k_weight, freq, kcache, vcache)
+    before the rotation (after the norm, when there is one).  ``per_head``: the norms take their
+    statistics head by head and their weights have one head's size.  ``key_skip``: the leading
+    elements of a key head that are neither normed nor weighted; with ``values_are_keys`` the values
+    are the elements behind them.  ``value_freq`` (32-bit, half a value head's size): every element of
+    a value head is turned before it is cached, pair m by position * value_freq[m], pairs
+    (m, m + dv/2) with ``value_pair_halves`` and (2m, 2m+1) without.  ``rotation_scale``: a factor on
+    the cosines and sines of the queries' and keys' rotation."""
+    _gpu(qkv, positions, token_req, block_table, q_weight, k_weight, freq, kcache, vcache, value_freq)
     _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qk_prepare: rows must be 2-d with unit inner stride")
     n = qkv.shape[0]
     dq = key_dim if query_dim is None else int(query_dim)
-    _need(not values_are_keys or value_dim == key_dim, "qk_prepare: values that are the keys have the keys' size")
+    key_skip = int(key_skip)
+    _need(not values_are_keys or value_dim == key_dim - key_skip, "qk_prepare: values that are the keys have the keys' size")
     need = nq * dq + (nkv * (key_dim + (0 if values_are_keys else value_dim)) if write_cache else 0)
     _need(qkv.shape[1] >= need, f"qk_prepare: rows of {qkv.shape[1]} hold no {need} elements")
     _i32(positions, "positions")
     _i32(token_req, "token_req")
     _need(positions.numel() == n and token_req.numel() == n, "positions/token_req must have one entry a token")
-    _f32_vector(q_weight, nq * dq, "qk_prepare: the query norm's weight")
-    _f32_vector(k_weight, nkv * key_dim, "qk_prepare: the key norm's weight")
+    _f32_vector(q_weight, dq if per_head else nq * dq, "qk_prepare: the query norm's weight")
+    _f32_vector(k_weight, (1 if per_head else nkv) * (key_dim - key_skip), "qk_prepare: the key norm's weight")
+    _f32_vector(value_freq, value_dim // 2, "qk_prepare: the values' frequencies")
     rot = 0
     if freq is not None:
         _need(freq.dim() == 1 and freq.dtype == torch.float32 and freq.is_contiguous() and 2 * freq.numel() <= min(key_dim, dq),
@@ -1218,7 +1334,9 @@ def qk_prepare(
          float(eps), freq.data_ptr() if freq is not None else None,
          kcache.data_ptr() if write_cache else None, vcache.data_ptr() if write_cache else None,
          n, nq, nkv if write_cache else 0, dq, key_dim, value_dim, rot, page_size, 1 if write_cache else 0,
-         1 if pair_halves else 0, 1 if values_are_keys else 0, _stream())
+         1 if pair_halves else 0, 1 if values_are_keys else 0, 1 if per_head else 0, key_skip,
+         value_freq.data_ptr() if value_freq is not None else None, 1 if value_pair_halves else 0, float(rotation_scale),
+         _stream())
 
 
 def gather_keys(kcache: torch.Tensor, block_table: torch.Tensor, req: torch.Tensor, pos: torch.Tensor, key_dim: int,
@@ -1266,6 +1384,7 @@ def attention_tile_f32(
     kv_len: torch.Tensor, tile_req: torch.Tensor, tile_row0: torch.Tensor, nq: int, nkv: int, key_dim: int,
     value_dim: int, page_size: int, heads_a_tile: int, window: int = 0, scale: float = 1.0,
     sink: torch.Tensor | None = None, split: bool | None = None, key_chunk: int = 0, longest: int = 0, first_row: int = 0,
+    score_bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Attention in 32-bit arithmetic on the matrix cores: every token of the step over its
     request's pages; ``tile_req`` / ``tile_row0`` name each tile's request and its first token's
@@ -1277,8 +1396,9 @@ def attention_tile_f32(
     depend on the batch): a split tile's keys are also cut at absolute multiples of ``key_chunk`` among
     workgroups, whose partial results a second kernel adds in ascending order.
     ``first_row``: ``q`` holds the step's rows from this one on only (the tiles name none before it), and so
-    does the result."""
-    _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink)
+    does the result.  ``score_bias``: sigmoid weights as in ``paged_attention_generic``."""
+    _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink, score_bias)
+    _f32_vector(score_bias, nq, "attention: the scores' biases")
     if split is None:
         split = tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) < ATTENTION_TILE_SPLIT_BELOW
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * key_dim,
@@ -1307,7 +1427,8 @@ def attention_tile_f32(
     call("tk_attention_tile_f32", dtype_code(q.dtype), q_base, q.stride(0), out_base, out.stride(0),
          kcache.data_ptr(), vcache.data_ptr(), block_table.data_ptr(), block_table.stride(0), q_start.data_ptr(),
          kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(), tile_req.numel(), nq, nkv, key_dim, value_dim,
-         page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None, int(heads_a_tile),
+         page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None,
+         score_bias.data_ptr() if score_bias is not None else None, int(heads_a_tile),
          1 if split else 0, int(key_chunk) if chunks else 0, chunks, part.data_ptr() if part is not None else None, _stream())
     return out
 
@@ -1428,11 +1549,13 @@ def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, e
 
 def post_norm_residual(x: torch.Tensor, branch: torch.Tensor, branch_weight: torch.Tensor, branch_eps: float,
                        weight: torch.Tensor | None = None, eps: float = 0.0, out_dtype: torch.dtype = torch.float32,
-                       in_place: bool = True) -> tuple[torch.Tensor, torch.Tensor | None]:
+                       in_place: bool = True, plain_rows: bool = False) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``x_new = x + branch / sqrt(mean(branch^2) + branch_eps) * branch_weight`` on a 32-bit
     stream (the branch 32-bit too), and, when ``weight`` is given, the rows of the norm that
     reads the new stream, ``x_new / sqrt(mean(x_new^2) + eps) * weight`` rounded once to
-    ``out_dtype``.  Returns (x_new, those rows or None).  ``in_place``: x_new overwrites x."""
+    ``out_dtype``.  Returns (x_new, those rows or None).  ``in_place``: x_new overwrites x.
+    ``plain_rows`` (without ``weight``): the rows returned are x_new itself rounded once to ``out_dtype``
+    (x_new when that is 32-bit): for sublayers that read the stream unnormed."""
     _gpu(x, branch, branch_weight, weight)
     _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "post_norm_residual: the stream must be contiguous float32 [rows, H]")
     _need(branch.shape == x.shape and branch.dtype == torch.float32 and branch.is_contiguous(),
@@ -1441,12 +1564,14 @@ def post_norm_residual(x: torch.Tensor, branch: torch.Tensor, branch_weight: tor
     _f32_vector(branch_weight, hidden, "post_norm_residual: the branch norm's weight")
     _f32_vector(weight, hidden, "post_norm_residual: a norm weight")
     x_out = x if in_place else torch.empty_like(x)
-    h = torch.empty((rows, hidden), dtype=out_dtype, device=x.device) if weight is not None else None
+    _need(not (plain_rows and weight is not None), "post_norm_residual: plain rows or a norm's rows, not both")
+    cast = plain_rows and out_dtype != torch.float32
+    h = torch.empty((rows, hidden), dtype=out_dtype, device=x.device) if (weight is not None or cast) else None
     if rows:
         call("tk_post_norm_residual", dtype_code(out_dtype), x.data_ptr(), branch.data_ptr(), branch_weight.data_ptr(),
              float(branch_eps), x_out.data_ptr(), weight.data_ptr() if weight is not None else None, float(eps),
              h.data_ptr() if h is not None else None, rows, hidden, _stream())
-    return x_out, h
+    return x_out, (x_out if plain_rows and not cast else h)
 
 
 def concat_cast(x: torch.Tensor, y: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

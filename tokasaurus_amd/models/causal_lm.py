@@ -28,6 +28,13 @@ class CausalLM:
         self.blocks = [build_with_shared(BLOCKS, b, self.shared) for b in spec.layers]
         self.head = build_with_shared(HEADS, spec.head, self.shared)
         self.connectors = [build_with_shared(CONNECTORS, c, self.shared) for c in spec.connectors]
+        # an embedding that can also write the rows of the first block's entry norm is told which norm that is
+        # (only one that merely rounds the stream: there is nothing of the norm to compute)
+        if hasattr(self.embedding, "reader") and spec.run_order and spec.run_order[0].before is None:
+            first = self.blocks[spec.run_order[0].layer]
+            entry = first.entry_norm() if first.fuses_norm else None
+            if getattr(entry, "plain_rows", False):
+                self.embedding.reader = entry
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
         self.weight_bytes = 0
@@ -60,6 +67,10 @@ class CausalLM:
     def state_needs(self) -> "list[StateNeed | None | list[StateNeed]]":
         return [_one_or_many(self.blocks[e.layer].state_needs()) for e in self.spec.run_order]
 
+    def embedding_state_need(self) -> "StateNeed | None":
+        """What the embedding keeps per request in its slot (``StepContext.embedding_state``), if anything."""
+        return self.embedding.state_need()
+
     # ---- one step
     def forward(
         self,
@@ -72,10 +83,10 @@ class CausalLM:
         """Run the batch of ``ctx`` and return logits [len(want_rows), vocab] in 32-bit;
         ``want_rows`` None stands for every row in order (no rows are picked out then).
         ``logits_out``: a contiguous buffer of that shape that receives the logits and is returned."""
-        x = self.embedding.forward(ctx)
+        # (an embedding may already have made the rows of the first block's entry norm)
+        x, prepared = stream_and_prepared(self.embedding.forward(ctx))
         order = self.spec.run_order
         last = len(order) - 1
-        prepared = None  # what a block has done for the norm that the next one (or the head) starts with
         # a connector reads the embedding's output again; blocks may update the stream in place
         x0 = x.clone() if self.connectors else None
         for i, entry in enumerate(order):

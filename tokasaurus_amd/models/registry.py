@@ -16,6 +16,8 @@ from tokasaurus_amd.models.kupuzen import kupuzen_spec
 from tokasaurus_amd.models.llama import llama_spec
 from tokasaurus_amd.config.taborax_config import TaboraxConfig
 from tokasaurus_amd.models.taborax import taborax_spec
+from tokasaurus_amd.config.sakevik_config import SakevikConfig
+from tokasaurus_amd.models.sakevik import sakevik_spec
 from tokasaurus_amd.models.spec import ModelSpec
 
 
@@ -41,6 +43,7 @@ def register_architecture(arch: Architecture, replace: bool = False) -> None:
 register_architecture(Architecture("llama", LlamaConfig.from_dict, llama_spec, class_names=("LlamaForCausalLM",)))
 register_architecture(Architecture("kupuzen", KupuzenConfig.from_dict, kupuzen_spec, class_names=("Kupuzen",)))
 register_architecture(Architecture("taborax", TaboraxConfig.from_dict, taborax_spec, class_names=("Taborax",)))
+register_architecture(Architecture("sakevik", SakevikConfig.from_dict, sakevik_spec, class_names=("Sakevik",)))
 
 
 def architecture_of(config_dict: dict[str, Any]) -> Architecture:

@@ -113,6 +113,7 @@ class StepContext:
     host_kv_len: list[int]
     host_slots: list[int]
     last_token: torch.Tensor | None = None  # [slots] int32, written by the sampler
+    embedding_state: torch.Tensor | None = None  # [slots + 1, ...]: what the embedding keeps per request, if anything
     max_q_len: int = 0
     max_kv_len: int = 0
     extras: dict[str, Any] = field(default_factory=dict)  # planning data of kernels, by name
@@ -260,7 +261,13 @@ class Embedding(Part):
     """From the step's token ids to the first residual stream [N, H] in the engine dtype.
     ``ctx.token_ids`` holds ids, or -(slot + 1) for a token to be read from ``ctx.last_token``."""
 
+    def state_need(self) -> "StateNeed | None":
+        """Per-request state of fixed size that the embedding keeps in the request's slot (an
+        embedding that reads the token before, say); it gets it as ``ctx.embedding_state``."""
+        return None
+
     def forward(self, ctx: StepContext) -> torch.Tensor:
+        """The stream, or (stream, ``Prepared``) when it has also made the rows of the first block's entry norm."""
         raise NotImplementedError
 
 

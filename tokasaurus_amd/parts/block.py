@@ -260,6 +260,77 @@ class SandwichNormBlock(Block):
         return x, Prepared(None, reader, h)
 
 
+@BLOCKS.register("post_norm")
+class PostNormBlock(Block):
+    """A norm behind every sublayer and none in front, on a 32-bit residual stream:
+        x <- x + post1(mixer(x));  x <- x + post2(ff(x))
+    ``feed_forward`` (with its norm) may be absent.  The sublayers read the stream itself, rounded once to
+    the storage type.  The branches hand over their last products' 32-bit sums; one kernel norms a
+    branch, adds it to the stream and writes the rows of whoever reads the new stream: the rounded stream
+    for this block's feed-forward or the next block of this kind, the normed rows for a norm (the
+    head's).  The post norms are ``stream_rmsnorm``s with plain weights; the mixer must have ``mix`` and
+    the feed-forward ``transform``."""
+
+    fuses_norm = True
+
+    def __init__(self, mixer: PartSpec, mixer_post_norm: PartSpec, feed_forward: PartSpec | None = None,
+                 ff_post_norm: PartSpec | None = None, shared: dict | None = None):
+        shared = shared if shared is not None else {}
+        if (feed_forward is None) != (ff_post_norm is None):
+            raise ValueError("a feed-forward and the norm behind it come together")
+        self.entry = build_with_shared(NORMS, PartSpec("stream_cast"), shared)
+        self.mixer = build_with_shared(MIXERS, mixer, shared)
+        self.mixer_post_norm = build_with_shared(NORMS, mixer_post_norm, shared)
+        self.feed_forward = build_with_shared(FEED_FORWARDS, feed_forward, shared) if feed_forward is not None else None
+        self.ff_post_norm = build_with_shared(NORMS, ff_post_norm, shared) if ff_post_norm is not None else None
+        for n in (self.mixer_post_norm, self.ff_post_norm):
+            if n is not None and (getattr(n, "same_rule", None) is None or n.unit_offset):
+                raise ValueError("a post_norm block takes stream_rmsnorm norms with plain weights")
+
+    def children(self) -> list[Part]:
+        return [c for c in (self.entry, self.mixer, self.mixer_post_norm, self.feed_forward, self.ff_post_norm) if c is not None]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [s for c in self.children() for s in c.tensor_specs()]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        for c in self.children():
+            c.load(tensors, placer)
+
+    def entry_norm(self):
+        return self.entry
+
+    def _add(self, x, branch, post, reader):
+        """Norm the branch, add it, and write the rows of ``reader``: the rounded stream for a reader that
+        only rounds, the normed rows for a plain-weight stream norm, nothing for any other."""
+        if getattr(reader, "plain_rows", False):
+            return ops.post_norm_residual(x, branch, post.weight, post.eps, out_dtype=self.entry.out_dtype, plain_rows=True)
+        return SandwichNormBlock._add(x, branch, post, reader)
+
+    def forward(self, x, ctx: StepContext, cache, state, rows, prepared: Prepared | None = None, next_norm=None):
+        if x.dtype != torch.float32:
+            raise TypeError("a post_norm block runs on a 32-bit stream (an embedding that writes one)")
+        if prepared is not None and prepared.normed is not None and getattr(prepared.norm, "plain_rows", False):
+            h = prepared.normed  # the rounded stream is the same whoever asked for it
+        else:
+            h = self.entry.forward(x)
+        a = self.mixer.mix(h, ctx, cache, state, rows, out_f32=True)
+        if rows is not None:
+            x = ops.gather_rows(x, rows)
+        tap = ctx.extras.get("stream_tap")
+        reader = self.entry if self.feed_forward is not None else next_norm
+        x, h = self._add(x, a, self.mixer_post_norm, reader)
+        if self.feed_forward is not None:
+            b = self.feed_forward.transform(h, out_f32=True)
+            reader = next_norm
+            x, h = self._add(x, b, self.ff_post_norm, reader)
+        if tap is not None:  # a list that collects the stream after every block (tests, debugging)
+            tap.append(x.clone())
+        if h is None or reader is None:
+            return x
+        return x, Prepared(None, reader, h)
+
+
 @CONNECTORS.register("embedding_mix")
 class EmbeddingMix(Connector):
     """x <- W [x; x0]: the stream and the embedding's output side by side through one matrix

@@ -59,3 +59,34 @@ class SquaredReLU(FeedForward):
 
     def transform(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
         return self.down(ops.squared_relu_(self.up(h)), out_f32=out_f32)
+
+
+@FEED_FORWARDS.register("clamped_glu")
+class ClampedGLU(FeedForward):
+    """A gated feed-forward with clamps: ``g = min(gate(h), limit)``, ``u = clamp(up(h), -limit, limit)``,
+    ``down(g * sigmoid(alpha * g) * (u + 1))``, no biases.  gate and up are one stacked product."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, names: dict[str, str], alpha: float = 1.702):
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.limit, self.alpha = float(limit), float(alpha)
+        if not self.limit > 0:
+            raise ValueError("the clamp's limit must be positive")
+        self.gate_up = Linear(hidden_size, [names["gate"], names["up"]], [intermediate_size] * 2)
+        self.down = Linear(intermediate_size, [names["down"]], [hidden_size])
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return self.gate_up.tensor_specs() + self.down.tensor_specs()
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.gate_up.load(tensors, placer)
+        self.down.load(tensors, placer)
+
+    def _inner(self, h: torch.Tensor) -> torch.Tensor:
+        return ops.clamped_glu(self.gate_up(h), self.limit, self.alpha)
+
+    def forward(self, h: torch.Tensor, residual: torch.Tensor):
+        return self.down(self._inner(h), residual=residual)
+
+    def transform(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
+        return self.down(self._inner(h), out_f32=out_f32)

@@ -6,7 +6,10 @@ learned sink per query head in the softmax's denominator (or one constant score 
 keys and values taken from another layer's cache (the run entry's ``cache_of``; the mixer then
 has no key and value tensors), a rotation that pairs the two halves of a head's leading part
 instead of neighbours, and values that are the keys themselves as projected, before the rotation
-(the mixer then has no value tensor).
+(the mixer then has no value tensor); biases on the projections; norms of queries and keys head by
+head with one weight for all heads; weights that are sigmoids of the biased scores instead of a
+softmax; values turned by their own position and the heads' results turned back by the query's; a
+sigmoid gate per head that reads the mixer's input.
 
 Scores, softmax weights, norms, angles and the rotation are 32-bit arithmetic in either storage
 type.  One kernel norms, rotates and appends (``ops.qk_prepare``); the attention itself runs on
@@ -76,6 +79,11 @@ class GroupedAttention(Mixer):
         sink_value: float | None = None,
         values_are_keys: bool = False,
         key_chunk: int = 0,
+        bias_names: dict[str, str] | None = None,
+        head_norm: dict | None = None,
+        score_bias_name: str | None = None,
+        value_rotation: dict | None = None,
+        gate_name: str | None = None,
     ):
         """``names``: checkpoint names of the q, k, v, o matrices (k and v only with ``own_kv``).
         ``projection_norm``: ``{"q": name, "k": name, "eps": eps}``, weights of the whole
@@ -86,8 +94,25 @@ class GroupedAttention(Mixer):
         tensor, every head's sink has this score (0: one is added to the softmax's denominator).
         ``values_are_keys``: ``names`` has no v; a token's values are its keys before the rotation.
         ``key_chunk``: in steps of few tokens a request's keys are cut at multiples of this many among
-        workgroups (0: never)."""
+        workgroups (0: never).  ``bias_names``: checkpoint names of biases under any of q, k, v, o.
+        ``head_norm``: ``{"q": name, "k": name, "eps": eps}``, RMS norms head by head with weights of one
+        head's size (instead of ``projection_norm``).  ``score_bias_name``: one number a query head; the
+        weight of a visible key is sigmoid(score + bias), not normalised over the keys (no softmax, no sink).
+        ``value_rotation``: ``{"base": b, "pair_halves": bool}``; the value at position j is cached turned,
+        pair m by j * b^(-2m/value_dim), and a head's result at position i is turned back by i.
+        ``gate_name``: a matrix [heads, hidden]; head h's result is multiplied by sigmoid(gate h)_h."""
         self.key_chunk = int(key_chunk)
+        bias_names = dict(bias_names or {})
+        self.head_norm = dict(head_norm) if head_norm else None
+        if self.head_norm and projection_norm:
+            raise ValueError("queries and keys are normed over the whole projection or head by head, not both")
+        self.score_bias_name = score_bias_name
+        if score_bias_name and (sink_name or sink_value is not None):
+            raise ValueError("sigmoid weights have no denominator for a sink to join")
+        self.value_rotation = dict(value_rotation) if value_rotation else None
+        if self.value_rotation and (values_are_keys or not own_kv or int(value_dim) % 2):
+            raise ValueError("turned values come with a value projection of the mixer's own and an even value size")
+        self.gate_name = gate_name
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
@@ -109,8 +134,15 @@ class GroupedAttention(Mixer):
         kv_sizes = [num_kv_heads * key_dim] + ([] if self.values_are_keys else [num_kv_heads * value_dim])
         kv_names = [names["k"]] + ([] if self.values_are_keys else [names["v"]])
         sizes = [num_heads * key_dim] + (kv_sizes if own_kv else [])
-        self.qkv = Linear(hidden_size, [names["q"]] + (kv_names if own_kv else []), sizes)
-        self.out = Linear(num_heads * value_dim, [names["o"]], [hidden_size])
+        stacked = [names["q"]] + (kv_names if own_kv else [])
+        biases = [bias_names.get("q")] + ([bias_names.get("k")] + ([] if self.values_are_keys else [bias_names.get("v")]) if own_kv else [])
+        if gate_name:  # the gate reads the same input: one more part of the stacked product
+            stacked, sizes, biases = stacked + [gate_name], sizes + [num_heads], biases + [None]
+        self.gate_col = sum(sizes) - num_heads if gate_name else None
+        self.qkv = Linear(hidden_size, stacked, sizes, bias_names=biases)
+        self.out = Linear(num_heads * value_dim, [names["o"]], [hidden_size], bias_names=[bias_names.get("o")])
+        self.score_bias: torch.Tensor | None = None
+        self.value_freq: torch.Tensor | None = None
         self.q_norm_weight: torch.Tensor | None = None
         self.k_norm_weight: torch.Tensor | None = None
         self.sink: torch.Tensor | None = None
@@ -128,8 +160,14 @@ class GroupedAttention(Mixer):
             specs.append(TensorSpec(self.projection_norm["q"], (self.num_heads * self.key_dim,), NORM_WEIGHT))
             if self.own_kv:
                 specs.append(TensorSpec(self.projection_norm["k"], (self.num_kv_heads * self.key_dim,), NORM_WEIGHT))
+        if self.head_norm:
+            specs.append(TensorSpec(self.head_norm["q"], (self.key_dim,), NORM_WEIGHT))
+            if self.own_kv:
+                specs.append(TensorSpec(self.head_norm["k"], (self.key_dim,), NORM_WEIGHT))
         if self.sink_name:
             specs.append(TensorSpec(self.sink_name, (self.num_heads,), VECTOR))
+        if self.score_bias_name:
+            specs.append(TensorSpec(self.score_bias_name, (self.num_heads,), VECTOR))
         return specs
 
     def cache_need(self) -> CacheNeed:
@@ -151,6 +189,16 @@ class GroupedAttention(Mixer):
             self.q_norm_weight = f32(self.projection_norm["q"])
             if self.own_kv:
                 self.k_norm_weight = f32(self.projection_norm["k"])
+        if self.head_norm:
+            self.q_norm_weight = f32(self.head_norm["q"])
+            if self.own_kv:
+                self.k_norm_weight = f32(self.head_norm["k"])
+        if self.score_bias_name:
+            self.score_bias = f32(self.score_bias_name)
+        if self.value_rotation:
+            dv, base = self.value_dim, float(self.value_rotation["base"])
+            self.value_freq = placer.place(("value_freq", dv, base), lambda: torch.tensor(
+                [base ** (-2.0 * m / dv) for m in range(dv // 2)], dtype=torch.float64).to(torch.float32).to(placer.device))
         if self.sink_name:
             self.sink = f32(self.sink_name)
         elif self.sink_value is not None:
@@ -165,24 +213,32 @@ class GroupedAttention(Mixer):
             raise RuntimeError("a mixer with key and value tensors of its own writes its cache; one without reads another's")
         nq, nkv, dk, dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         qkv = self.qkv(h)
-        eps = float(self.projection_norm["eps"]) if self.projection_norm else 0.0
+        normed = self.projection_norm or self.head_norm
+        eps = float(normed["eps"]) if normed else 0.0
+        v_halves = bool(self.value_rotation and self.value_rotation.get("pair_halves"))
         ops.qk_prepare(qkv, ctx.positions, ctx.token_req, cache.block_table, self.q_norm_weight,
                        self.k_norm_weight if self.own_kv else None, eps,
                        self.position.freq if self.position is not None else None,
                        cache.keys, cache.values, nq, nkv, dk, dv, cache.page_size, write_cache=self.own_kv,
                        pair_halves=self.position is not None and self.position.pair_halves,
-                       values_are_keys=self.values_are_keys)
+                       values_are_keys=self.values_are_keys, per_head=self.head_norm is not None,
+                       value_freq=self.value_freq, value_pair_halves=v_halves,
+                       rotation_scale=self.position.magnitude if self.position is not None else 1.0)
         if ops.attention_tile_f32_fits(nq, nkv, dk, dv, cache.page_size):
             gg = ops.attention_tile_heads(nq // nkv, ctx.max_q_len)
             tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
             attn = ops.attention_tile_f32(qkv, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
                                           tile_req, tile_row0, nq, nkv, dk, dv, cache.page_size, gg,
                                           window=self.window, scale=self.scale, sink=self.sink, key_chunk=self.key_chunk,
-                                          longest=ctx.extras.get("kv_bound", ctx.max_kv_len))
+                                          longest=ctx.extras.get("kv_bound", ctx.max_kv_len), score_bias=self.score_bias)
         else:  # sizes that the matrix-core kernel does not take
             attn = ops.paged_attention_generic(qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
                                                nq, nkv, dk, cache.page_size, window=self.window, scale=self.scale,
-                                               value_dim=dv, sink=self.sink)
+                                               value_dim=dv, sink=self.sink, score_bias=self.score_bias)
+        if self.value_freq is not None or self.gate_col is not None:
+            # the heads' results turned back by their own positions, then each head's gate
+            gate = qkv[:, self.gate_col : self.gate_col + nq] if self.gate_col is not None else None
+            ops.unrotate_gate_(attn, ctx.positions, self.value_freq, v_halves, gate, nq, dv)
         return attn if rows is None else ops.gather_rows(attn, rows)
 
     def mix(self, h, ctx, cache, state, rows, out_f32: bool = False):

@@ -68,3 +68,22 @@ class StreamRMSNorm(Norm):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.residual_norm(x, weights=(self.weight, None), unit_offset=self.unit_offset, eps=self.eps,
                                  out_dtype=self.out_dtype)[1]
+
+
+@NORMS.register("stream_cast")
+class StreamCast(Norm):
+    """No norm at all: the 32-bit stream rounded once to the storage type, for sublayers that read
+    the stream itself (blocks that norm a sublayer's output only).  It stands where a norm would, so that
+    the pass that updates the stream can write its rows like any other reader's (``plain_rows``)."""
+
+    fusable_rms = False
+    plain_rows = True
+
+    def __init__(self):
+        self.out_dtype: torch.dtype | None = None
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.out_dtype = placer.dtype
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.cast_rows(x, self.out_dtype)

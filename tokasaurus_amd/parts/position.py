@@ -87,6 +87,28 @@ def interleaved_frequencies(dims: int, base: float, scaling: dict | None) -> tor
     return torch.tensor(out, dtype=torch.float64).to(torch.float32)
 
 
+def ramp_frequencies(dims: int, base: float, ramp: dict) -> tuple[torch.Tensor, float]:
+    """Frequencies blended between f_i = base^(-2i/dims) and f_i / factor by a ramp over the pair's
+    index (``ramp``: ``factor``, ``original``, ``fast``, ``slow``), and the factor that goes on cosine and
+    sine.  With index(t) = dims ln(original / (2 pi t)) / (2 ln base), the pair whose wavelength makes t
+    turns over ``original`` positions: lo = max(floor(index(fast)), 0), hi = min(ceil(index(slow)),
+    dims - 1), r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1); the frequency is
+    f_i / factor * r_i + f_i (1 - r_i) and the factor 0.1 ln(factor) + 1.  64-bit on the host, rounded once."""
+    factor, original = float(ramp["factor"]), float(ramp["original"])
+
+    def index(turns: float) -> float:
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+    lo = max(math.floor(index(float(ramp["fast"]))), 0)
+    hi = min(math.ceil(index(float(ramp["slow"]))), dims - 1)
+    out = []
+    for i in range(dims // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        out.append(f / factor * r + f * (1.0 - r))
+    return torch.tensor(out, dtype=torch.float64).to(torch.float32), 0.1 * math.log(factor) + 1.0
+
+
 @POSITION_ENCODINGS.register("rotary_interleaved")
 class InterleavedRotary(PositionEncoding):
     """A rotation of neighbouring elements (2i, 2i+1) of the leading ``dims`` elements of a head
@@ -95,17 +117,27 @@ class InterleavedRotary(PositionEncoding):
 
     pair_halves = False  # which elements form a pair: neighbours (2i, 2i+1), or (i, i + dims/2)
 
-    def __init__(self, dims: int, base: float, scaling: dict | None = None):
+    def __init__(self, dims: int, base: float, scaling: dict | None = None, ramp: dict | None = None):
+        """``scaling``: rescaling by wavelength bands (``interleaved_frequencies``); ``ramp``: a blend by
+        the pair's index with a factor on cosine and sine (``ramp_frequencies``); at most one of them."""
         if dims % 2 or dims <= 0:
             raise ValueError(f"a rotation of pairs needs an even number of elements, got {dims}")
+        if scaling and ramp:
+            raise ValueError("a rotation is rescaled by bands of wavelength or by a ramp, not both")
         self.dims = int(dims)
         self.base = float(base)
         self.scaling = dict(scaling) if scaling else None
+        self.ramp = dict(ramp) if ramp else None
+        self.magnitude = 1.0  # what cosine and sine are multiplied by
         self.freq: torch.Tensor | None = None
 
     def prepare(self, device: torch.device) -> None:
         if self.freq is None:
-            self.freq = interleaved_frequencies(self.dims, self.base, self.scaling).to(device)
+            if self.ramp:
+                freq, self.magnitude = ramp_frequencies(self.dims, self.base, self.ramp)
+                self.freq = freq.to(device)
+            else:
+                self.freq = interleaved_frequencies(self.dims, self.base, self.scaling).to(device)
 
 
 @POSITION_ENCODINGS.register("rotary_halves")
