@@ -82,7 +82,7 @@ def parse() -> argparse.Namespace:
                    help="instead of the decode steps, a case that shapes of one length do not show (prints its own line): "
                         "chunked-prefill: one prompt of --context tokens in portions of --portion tokens; "
                         "mixed-decode: decode steps of --batch - 1 requests of --short tokens beside one of --context tokens")
-    p.add_argument("--design", default=None, choices=["kupuzen", "taborax"],
+    p.add_argument("--design", default=None, choices=["kupuzen", "taborax", "sakevik"],
                    help="instead of the decode steps: prefill and decode of this design at layer sizes of --design-sizes "
                         "beside the Llama shape of equal width, heads, feed-forward and layers (prints its own line)")
     p.add_argument("--design-sizes", default="1b,3b", help="which sizes of DESIGN_SIZES, comma separated")
@@ -386,6 +386,30 @@ def taborax_like(size: dict, layers: int) -> dict:
             "loop": {"start": 1, "stop": 3, "times": 2}, "layers": made}
 
 
+# A Sakevik of the same width, vocabulary, feed-forward and number of layers: in every four layers two of attention
+# with sigmoid weights (the Llama heads, half of each rotated, turned values, a window of 1,024 keys), one of latent
+# attention (the Llama heads of the Llama size beside a rotated part of 64, over a latent of 192: a cached key of 256, a
+# window of 1,024 keys, the ramp between frequency scales) and one recurrence of twice the width without a feed-forward.
+def sakevik_like(size: dict, layers: int) -> dict:
+    ll = size["llama"]
+    d = ll["hidden_size"] // ll["num_attention_heads"]
+    ff = {"kind": "dense", "ff": ll["intermediate_size"], "limit": 7.0}
+    attention = {"type": "attention", "mlp": ff, "mixer": {
+        "heads": ll["num_attention_heads"], "kv_heads": ll["num_key_value_heads"], "dim": d, "vdim": d, "scale": d ** -0.5,
+        "mask": {"size": size["window"]}, "rot": {"base": ll["rope_theta"], "dims": d // 2}}}
+    latent = {"type": "latent_attention", "mlp": ff, "mixer": {
+        "heads": ll["num_attention_heads"], "dim": d, "rot_dim": 64, "vdim": d, "kv_rank": 192, "scale": (d + 64) ** -0.5,
+        "mask": {"size": size["window"]},
+        "rot": {"base": ll["rope_theta"], "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}}
+    gru = {"type": "mingru", "mlp": None, "mixer": {"width": 2 * ll["hidden_size"]}}
+    return {"architecture": "Sakevik", "vocab": ll["vocab_size"], "width": ll["hidden_size"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": float(ll["hidden_size"]) ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "logit_scale": 0.5, "layers": [(attention, latent, gru, attention)[i % 4] for i in range(layers)]}
+
+
+DESIGN_MODELS = {"kupuzen": kupuzen_like, "taborax": taborax_like, "sakevik": sakevik_like}
+
+
 def run_design(args) -> int:
     """Prefill of one prompt and decode steps of the new design beside the Llama shape of equal
     size, both with seeded random weights through the same runner and engine."""
@@ -398,7 +422,7 @@ def run_design(args) -> int:
     for name in [x for x in args.design_sizes.split(",") if x]:
         size = DESIGN_SIZES[name]
         configs = {"llama": dict(size["llama"], num_hidden_layers=args.design_layers),
-                   args.design: (kupuzen_like if args.design == "kupuzen" else taborax_like)(size, args.design_layers)}
+                   args.design: DESIGN_MODELS[args.design](size, args.design_layers)}
         if args.design_only:
             del configs["llama"]
         rec = {}
