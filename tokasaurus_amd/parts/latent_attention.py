@@ -156,9 +156,10 @@ class LatentAttention(Mixer):
                 self.expand.load(tensors, placer)
             else:
                 def expansion() -> torch.Tensor:
-                    w = torch.zeros((H * (dr + d) + H * dv, dr + r), dtype=placer.dtype)
+                    where = tensors[n["uk"]].device
+                    w = torch.zeros((H * (dr + d) + H * dv, dr + r), dtype=placer.dtype, device=where)
                     keys = w[: H * (dr + d)].view(H, dr + d, dr + r)
-                    keys[:, :dr, :dr] = torch.eye(dr, dtype=placer.dtype)
+                    keys[:, :dr, :dr] = torch.eye(dr, dtype=placer.dtype, device=where)
                     keys[:, dr:, dr:] = tensors[n["uk"]].to(placer.dtype).view(H, d, r)
                     w[H * (dr + d) :, dr:] = tensors[n["uv"]].to(placer.dtype)
                     return w.contiguous().to(placer.device)
@@ -166,8 +167,9 @@ class LatentAttention(Mixer):
                 self.expand_cached.weight = placer.place(("expansion_with_rotated_part", n["uk"], n["uv"]), expansion)
 
         def to_latent() -> torch.Tensor:
-            w = torch.zeros((H, dr + r, dr + d), dtype=placer.dtype)
-            w[:, :dr, :dr] = torch.eye(dr, dtype=placer.dtype)
+            where = tensors[n["uk"]].device
+            w = torch.zeros((H, dr + r, dr + d), dtype=placer.dtype, device=where)
+            w[:, :dr, :dr] = torch.eye(dr, dtype=placer.dtype, device=where)
             w[:, dr:, dr:] = tensors[n["uk"]].to(placer.dtype).view(H, d, r).transpose(1, 2)
             return w.contiguous().to(placer.device)
 

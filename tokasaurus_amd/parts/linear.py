@@ -73,7 +73,8 @@ class Linear:
         self.weight = placer.place(("row_major", *self.names), make)
         if self.bias_names is not None:
             def make_bias() -> torch.Tensor:
-                parts = [tensors[b].to(placer.dtype) if b is not None else torch.zeros((o,), dtype=placer.dtype)
+                where = next(tensors[b].device for b in self.bias_names if b is not None)
+                parts = [tensors[b].to(placer.dtype) if b is not None else torch.zeros((o,), dtype=placer.dtype, device=where)
                          for b, o in zip(self.bias_names, self.out_features)]
                 return torch.cat(parts).contiguous().to(placer.device)
 
