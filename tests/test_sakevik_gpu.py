@@ -66,8 +66,10 @@ def test_recurrence_kernel(width, lens):
         starts.append(starts[-1] + l)
     q_start = torch.tensor(starts, dtype=torch.int32, device=dev)
     state = state0.clone()
-    out = ops.min_gru(proj, state, q_start, slots, width, max(lens), torch.float32)
+    bias = torch.randn(2 * width, device=dev)
+    out = ops.min_gru(proj, state, q_start, slots, width, max(lens), torch.float32, bias=bias)
     p = proj.double().cpu()
+    p[:, : 2 * width] += bias.double().cpu()
     for r, l in enumerate(lens):
         S = state0[int(slots[r])].double().cpu()
         for t in range(starts[r], starts[r + 1]):
@@ -81,8 +83,10 @@ def test_recurrence_kernel(width, lens):
     if len(lens) == 1 and lens[0] > 9:
         st = state0.clone()
         one = torch.tensor([int(slots[0])], dtype=torch.int32, device=dev)
-        a = ops.min_gru(proj[:9], st, torch.tensor([0, 9], dtype=torch.int32, device=dev), one, width, 9, torch.float32)
-        b = ops.min_gru(proj[9:], st, torch.tensor([0, n - 9], dtype=torch.int32, device=dev), one, width, n - 9, torch.float32)
+        a = ops.min_gru(proj[:9], st, torch.tensor([0, 9], dtype=torch.int32, device=dev), one, width, 9, torch.float32, bias=bias)
+        b = ops.min_gru(proj[9:12], st, torch.tensor([0, 3], dtype=torch.int32, device=dev), one, width, 3, torch.float32, bias=bias)
+        b = torch.cat([b, ops.min_gru(proj[12:], st, torch.tensor([0, n - 12], dtype=torch.int32, device=dev), one, width, n - 12,
+                                      torch.float32, bias=bias)])
         assert torch.equal(torch.cat([a, b]), out) and torch.equal(st, state)
 
 

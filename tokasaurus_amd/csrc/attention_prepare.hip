@@ -76,21 +76,23 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   const int nqe = nq * dq, nke = nkv * dk;
   float rq = 1.f, rk = 1.f;
   if (per_head) {
-    // a wavefront a head: 1 / rms of the head's own elements (the key's behind k_skip)
-    const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE, waves = blockDim.x / TK_WAVE;
+    // sixteen lanes a head: 1 / rms of the head's own elements (the key's behind k_skip)
+    const int sub = threadIdx.x & 15, team = threadIdx.x >> 4, teams = blockDim.x >> 4;
     const int heads = nq + (write_cache ? nkv : 0);
-    for (int h = wave; h < heads; h += waves) {
+    for (int h = team; h < heads; h += teams) {
       const bool is_q = h < nq;
       const T* src = is_q ? row + (size_t)h * dq : row + nqe + (size_t)(h - nq) * dk + k_skip;
       const int n = is_q ? dq : dk - k_skip;
+      const bool normed = is_q ? q_weight != nullptr : k_weight != nullptr;
       float ss = 0.f;
-      if (is_q ? q_weight != nullptr : k_weight != nullptr)
-        for (int i = lane; i < n; i += TK_WAVE) {
+      if (normed)
+        for (int i = sub; i < n; i += 16) {
           const float v = to_f32<T>(src[i]);
           ss = fmaf(v, v, ss);
         }
-      ss = wave_sum(ss);
-      if (lane == 0) head_r[h] = (is_q ? q_weight != nullptr : k_weight != nullptr) ? 1.0f / sqrtf(ss / (float)n + eps) : 1.f;
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, TK_WAVE);  // (stays inside the sixteen lanes)
+      if (sub == 0) head_r[h] = normed ? 1.0f / sqrtf(ss / (float)n + eps) : 1.f;
     }
   } else if (q_weight) {
     float ss = 0.f;

@@ -72,6 +72,9 @@ struct GemmArgs {
   bf16_t* vcache;  // [page][kv head] pages of values
   int nq, nkv, d, P;
   const bf16_t* bias;  // [rows of W] or null: added to the product before the epilogue
+  // the gated epilogue's other form (glu_limit > 0): g = min(gate, limit), u = clamp(up, -limit, limit),
+  // g * sigmoid(glu_alpha * g) * (u + 1), 32-bit until the one rounding at the store
+  float glu_limit, glu_alpha;
   int M, N, K;  // N: outputs (for SwiGLU the intermediate size; W then has 2N rows, gate first)
   int TH;       // weight rows of a tile that are used (16, or 8 to make twice the workgroups of a narrow output)
 };
@@ -88,8 +91,17 @@ __device__ __forceinline__ void store4(const GemmArgs& a, f32x4_t v, f32x4_t up,
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     o[j] = v[j] * scale + bias_at(a, n + j, a.N);
-    if (EPI == EPI_SWIGLU)
-      o[j] = silu_mul_bf16(v[j] * scale + bias_at(a, n + j, a.N), up[j] * scale + bias_at(a, a.N + n + j, 2 * a.N));
+    if (EPI == EPI_SWIGLU) {
+      const float g = v[j] * scale + bias_at(a, n + j, a.N), u = up[j] * scale + bias_at(a, a.N + n + j, 2 * a.N);
+      if (a.glu_limit > 0.f) {
+        // (the operands rounded to the storage type first, as the separate kernel behind a product finds them)
+        const float gc = fminf(round_to<bf16_t>(g), a.glu_limit);
+        const float uc = fminf(fmaxf(round_to<bf16_t>(u), -a.glu_limit), a.glu_limit);
+        o[j] = gc / (1.0f + expf(-a.glu_alpha * gc)) * (uc + 1.0f);
+      } else {
+        o[j] = silu_mul_bf16(g, u);
+      }
+    }
     if (EPI == EPI_RESIDUAL && n + j < a.N)
       o[j] = round_to<bf16_t>(o[j]) + __bfloat162float(a.residual[(size_t)token * a.ldr + n + j]);
   }
@@ -673,6 +685,8 @@ struct GemmExtra {
   int nq, nkv, d, P;
   // a bias, one value a row of W, of the storage type
   const void* bias;
+  // the gated epilogue with clamps (see GemmArgs); 0: the plain one
+  float glu_limit, glu_alpha;
 };
 
 // Number of partial sums a row gets from the residual epilogue with emit_w: one a tile.
@@ -750,6 +764,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
     a.kcache = (bf16_t*)extra->kcache; a.vcache = (bf16_t*)extra->vcache;
     a.nq = extra->nq; a.nkv = extra->nkv; a.d = extra->d; a.P = extra->P;
     a.bias = (const bf16_t*)extra->bias;
+    a.glu_limit = extra->glu_limit; a.glu_alpha = extra->glu_alpha;
     norm = a.sumsq_in != nullptr;
   }
   TK_REQUIRE(!norm || a.parts_in > 0, "gemm_skinny: a norm in front needs its partial sums");

@@ -43,7 +43,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_softcap": [_P, c_size_t, c_float, _P],
         "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 13 + [_P, c_int, c_float, _P],
         "tk_unrotate_gate": [c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P],
-        "tk_min_gru": [c_int, _P, c_int, _P, c_size_t, _P, _P, _P, c_int, c_int, c_int, _P],
+        "tk_min_gru": [c_int, _P, c_int, _P, _P, c_size_t, _P, _P, _P, c_int, c_int, c_int, _P],
         "tk_embed_bigram": [c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P],
         "tk_cast_rows": [c_int, _P, _P, c_size_t, _P],
         "tk_scale_values": [_P, c_size_t, c_float, _P],

@@ -838,7 +838,7 @@ class _GemmExtra(ctypes.Structure):
         ("table_stride", ctypes.c_int), ("cos_t", ctypes.c_void_p), ("sin_t", ctypes.c_void_p),
         ("kcache", ctypes.c_void_p), ("vcache", ctypes.c_void_p),
         ("nq", ctypes.c_int), ("nkv", ctypes.c_int), ("d", ctypes.c_int), ("P", ctypes.c_int),
-        ("bias", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p), ("glu_limit", ctypes.c_float), ("glu_alpha", ctypes.c_float),
     ]
 
 
@@ -886,6 +886,7 @@ def gemm_skinny_bf16(
     out: torch.Tensor | None = None,
     bias: torch.Tensor | None = None,
     fold: bool = True,
+    glu: tuple[float, float] | None = None,
 ):
     """a [M <= 128, K] times w [N, K] transposed on the matrix cores, with the
     epilogue fused: + residual, 32-bit output, (``swiglu``: w is [gate | up]
@@ -897,6 +898,8 @@ def gemm_skinny_bf16(
     (with ``residual``): the weight of the norm that follows; returns
     ``(out, Prenorm)`` for it.  ``out``: where the result goes instead of new memory.
     ``bias`` (one value a row of ``w``): added to the product before the epilogue.
+    ``glu`` (with ``swiglu``): (limit, alpha); the gated epilogue is then min(gate, limit) *
+    sigmoid(alpha * min(gate, limit)) * (clamp(up, -limit, limit) + 1).
     ``waves_k``, ``tiles``, ``staged``, ``tile_rows``, ``fold``: the kernel's own choices overridden (for measurements)."""
     _gpu(a, w, residual, emit_weight, bias)
     _check_bias(bias, w, "gemm_skinny")
@@ -914,6 +917,10 @@ def gemm_skinny_bf16(
         n //= 2
         n_out = n
         epi = EPI_SWIGLU
+        if glu is not None:
+            _need(glu[0] > 0, "gemm_skinny: the clamp's limit must be positive")
+            extra.glu_limit, extra.glu_alpha = float(glu[0]), float(glu[1])
+            use_extra = True
     elif rope is not None:
         _need(residual is None and not out_f32, "gemm_skinny: the rotation epilogue stands alone")
         epi = EPI_ROPE
@@ -1222,12 +1229,14 @@ def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tens
 
 
 def min_gru(proj: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, slots: torch.Tensor, width: int, longest: int,
-            out_dtype: torch.dtype) -> torch.Tensor:
+            out_dtype: torch.dtype, bias: torch.Tensor | None = None) -> torch.Tensor:
     """The gated recurrence ``S <- (1 - z) S + z cand`` per channel over every request's tokens of this
     step, from and to the request's slot of ``state`` [slots, width] (32-bit): ``proj`` holds the 32-bit
     sums [a | u | g] ([tokens, 3 width]; z = sigmoid(a), cand = u + 1/2 for u >= 0 and sigmoid(u) below);
-    returns S_t * silu(g) rounded once to ``out_dtype``.  ``longest``: the most tokens a request brings."""
-    _gpu(proj, state, q_start, slots)
+    returns S_t * silu(g) rounded once to ``out_dtype``.  ``longest``: the most tokens a request brings.
+    ``bias`` (32-bit, [2 width]): added to a and to u here, when the product has not."""
+    _gpu(proj, state, q_start, slots, bias)
+    _f32_vector(bias, 2 * width, "min_gru: the biases of z and of the candidate")
     _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1 and proj.shape[1] >= 3 * width,
           "min_gru: 32-bit rows [a | u | g]")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.stride(1) == 1 and state.shape[1] >= width,
@@ -1236,7 +1245,8 @@ def min_gru(proj: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, slot
     _i32(slots, "slots")
     _need(q_start.numel() == slots.numel() + 1, "min_gru: one slot a request")
     out = torch.empty((proj.shape[0], width), dtype=out_dtype, device=proj.device)
-    call("tk_min_gru", dtype_code(out_dtype), proj.data_ptr(), proj.stride(0), state.data_ptr(), state.stride(0), q_start.data_ptr(),
+    call("tk_min_gru", dtype_code(out_dtype), proj.data_ptr(), proj.stride(0), bias.data_ptr() if bias is not None else None,
+         state.data_ptr(), state.stride(0), q_start.data_ptr(),
          slots.data_ptr(), out.data_ptr(), slots.numel(), int(width), int(longest), _stream())
     return out
 

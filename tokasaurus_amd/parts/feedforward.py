@@ -83,7 +83,7 @@ class ClampedGLU(FeedForward):
         self.down.load(tensors, placer)
 
     def _inner(self, h: torch.Tensor) -> torch.Tensor:
-        return ops.clamped_glu(self.gate_up(h), self.limit, self.alpha)
+        return self.gate_up(h, swiglu=True, glu=(self.limit, self.alpha))
 
     def forward(self, h: torch.Tensor, residual: torch.Tensor):
         return self.down(self._inner(h), residual=residual)

@@ -99,6 +99,7 @@ class Linear:
         rows: int | None = None,
         swiglu: bool = False,
         out: torch.Tensor | None = None,
+        glu: tuple[float, float] | None = None,
     ) -> torch.Tensor:
         """x [M, in] -> [M, out].  ``residual``: returns residual + product (the
         product rounded to the storage type first).  ``out_f32``: 32-bit output.
@@ -106,7 +107,9 @@ class Linear:
         ``rows`` limits the product to the first output rows of the stacked
         weight (a mixer that only needs its queries).  ``x`` may be a ``Normed``:
         the norm is folded into the product when it was prepared, else applied first.
-        ``out`` (with ``out_f32``): a buffer [M, out] for the result, in place of new memory."""
+        ``out`` (with ``out_f32``): a buffer [M, out] for the result, in place of new memory.
+        ``glu`` (with ``swiglu``): (limit, alpha) of the gated activation with clamps, in place of silu(gate) * up."""
+        gated = (lambda p: ops.clamped_glu(p, glu[0], glu[1])) if glu is not None else ops.swiglu
         assert out is None or (out_f32 and residual is None and not swiglu), "a result buffer goes with 32-bit output only"
         w, bias = self.weight, self.bias
         if rows is not None and rows != self.total_out:
@@ -123,7 +126,7 @@ class Linear:
         if w.dtype == torch.bfloat16 and m > 0 and (m > ops.SKINNY_ROWS or self._aligned()):
             if self._fast(m, swiglu, out_f32):
                 return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu,
-                                            prenorm=prenorm, norm_eps=eps, out=out, bias=bias)
+                                            prenorm=prenorm, norm_eps=eps, out=out, bias=bias, glu=glu if swiglu else None)
             # library matrix product (hipBLASLt), 32-bit accumulation; with a bias through the tensor
             # library, whose call adds it to the 32-bit sums in the product's own epilogue (addmm)
             direct = ops.gemm_library_direct(x, w)
@@ -142,10 +145,10 @@ class Linear:
                 # the product is rounded to the storage type before the residual is added, as in the
                 # few-row kernel and in the pass that adds and norms (and as the reference's separate add)
                 return ops.add(prod, residual.contiguous())
-            return ops.swiglu(prod) if swiglu else prod
+            return gated(prod) if swiglu else prod
         # the 32-bit path, and few bfloat16 rows of a width the matrix-core kernel does not take
         prod = ops.gemm_generic(x, w, residual=residual, out_f32=out_f32, out=out, bias=bias)
-        return ops.swiglu(prod) if swiglu else prod
+        return gated(prod) if swiglu else prod
 
     def with_residual(
         self, x: torch.Tensor, residual: torch.Tensor, emit_norm: Norm | None
