@@ -22,6 +22,23 @@
 #include "common.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+
+// Scores from bfloat16 storage: the product of two bfloat16 numbers is exact in 32-bit, so the matrix cores'
+// bfloat16 product with 32-bit sums (v_mfma_f32_16x16x32_bf16) gives 32-bit scores of the stored queries and keys
+// like the 32-bit product of the converted operands, at an eighth of the instructions and without the conversions.
+// Its operands are what a lane holds anyway: 8 neighbouring elements of key lane % 16 (of the column's query) from
+// element 8 * (lane / 16) of every 32 on.  The weighted values stay 32-bit products: the weights are 32-bit numbers.
+template <typename T>
+struct ScoresFromStorage { static constexpr bool value = false; };
+template <>
+struct ScoresFromStorage<bf16_t> { static constexpr bool value = true; };
+template <typename R>
+__device__ __forceinline__ bf16x8_t as_bf16x8(const R& raw) {
+  bf16x8_t v;
+  __builtin_memcpy(&v, &raw, sizeof(v));
+  return v;
+}
 
 #define AT_WAVES 4
 #define AT_MAX_KM 8   // dk <= 256
@@ -78,15 +95,22 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   const int pieces = dk / 8;
   const size_t key_page = key_page_elems(P, dk);
 
-  // the column's query, piece c + 4 m
-  float qv[KM][8];
+  // the column's query, piece c + 4 m (as stored, for scores from storage; else as 32-bit numbers)
+  constexpr bool STORED = ScoresFromStorage<T>::value;
+  float qv[STORED ? 1 : KM][8];
+  Raw8<T> qraw[STORED ? KM : 1];
 #pragma unroll
   for (int m = 0; m < KM; ++m) {
     const int piece = c + 4 * m;
     const bool in = live && piece < pieces;
     const T* src = q + (size_t)(in ? tok : 0) * q_stride + (size_t)head * dk + (in ? piece : 0) * 8;
+    if constexpr (STORED) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qv[m][e] = in ? to_f32<T>(src[e]) : 0.f;
+      for (int e = 0; e < 8; ++e) qraw[m].v[e] = in ? src[e] : from_f32<T>(0.f);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qv[m][e] = in ? to_f32<T>(src[e]) : 0.f;
+    }
   }
 
   v4f o[VT];
@@ -160,11 +184,17 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     }
     // S^T = K Q^T (a piece beyond the head's size meets zeros of the query)
     v4f s = (v4f){0.f, 0.f, 0.f, 0.f};
+    if constexpr (STORED) {
 #pragma unroll
-    for (int m = 0; m < KM; ++m)
+      for (int m = 0; m < KM; ++m)
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kr[m]), as_bf16x8(qraw[m]), s, 0, 0, 0);
+    } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        s = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32<T>(kr[m].v[e]), qv[m][e], s, 0, 0, 0);
+      for (int m = 0; m < KM; ++m)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          s = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32<T>(kr[m].v[e]), qv[m][e], s, 0, 0, 0);
+    }
     // this lane now holds, for its column, keys k0 + 4 c + i
     float sc[4];
     float tmax = -INFINITY;
