@@ -89,8 +89,12 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   const int pos0 = kv - (q_end - row0);         // position of the tile's first token
   const int pos = pos0 + col / gg;              // of this column's token
   const int last_all = pos0 + n_tok - 1;  // the last key any column of the tile sees
-  const int last = PART ? min(last_all, ((int)blockIdx.z + 1) * chunk - 1) : last_all;  // the last this workgroup walks
-  const int lo_tile = max(window > 0 ? max(0, pos0 - window + 1) : 0, PART ? (int)blockIdx.z * chunk : 0);
+  // (PART) this workgroup's chunk: with a window the launch holds only as many chunks as a window touches, and
+  // blockIdx.z counts from the chunk of the first key that the tile sees (absolute multiples of `chunk` all the same)
+  const int first_seen = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int zc = PART ? first_seen / chunk + (int)blockIdx.z : 0;
+  const int last = PART ? min(last_all, (zc + 1) * chunk - 1) : last_all;  // the last this workgroup walks
+  const int lo_tile = max(first_seen, PART ? zc * chunk : 0);
   const int* table = block_table + (size_t)r * table_stride;
   const int pieces = dk / 8;
   const size_t key_page = key_page_elems(P, dk);

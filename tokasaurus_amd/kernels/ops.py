@@ -1426,9 +1426,15 @@ def attention_tile_f32(
         # longer chunks where the step has workgroups enough without short ones: a chunk's walk should be long
         # enough to hide its first loads
         groups = tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile))
-        while key_chunk < ATTENTION_TILE_LONGEST_CHUNK and groups * -(-int(longest) // (2 * key_chunk)) >= ATTENTION_TILE_WORKGROUPS:
+        # (behind a window a tile sees at most window + 15 keys, whatever the request's length: they lie in
+        # `seen // chunk + 1` chunks at most, one more when they start inside one, and the kernel counts a tile's
+        # chunks from the first it sees)
+        seen = min(int(longest), int(window) + 15) if window > 0 else int(longest)
+        while key_chunk < ATTENTION_TILE_LONGEST_CHUNK and groups * -(-seen // (2 * key_chunk)) >= ATTENTION_TILE_WORKGROUPS:
             key_chunk *= 2
         chunks = -(-int(longest) // int(key_chunk))
+        if window > 0:
+            chunks = min(chunks, -(-seen // int(key_chunk)) + 1)
         words = load("core").tk_attention_tile_part_words(value_dim)
         part = torch.empty((tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) * chunks * words,), dtype=torch.float32, device=q.device)
     # the kernel finds a tile's rows by their place in the step
