@@ -50,6 +50,27 @@ struct __align__(16) Raw8 { T v[8]; };
 template <typename T>
 struct __align__(sizeof(T) * 4) Raw4 { T v[4]; };
 
+// What may follow the weighted sum of the values before it is stored, for mixers whose values were turned by their own
+// positions and whose heads have a gate: pair m of a head's result is turned back by -position * vfreq[m] (pairs
+// (m, m + dv/2) with `pair_half`, which the launch takes only where dv is 16 times the kernel's VT, and (2m, 2m + 1)
+// without), then the head is multiplied by sigmoid(gate[token][head]).  Null pointers: nothing of the kind.
+template <typename T>
+struct AfterSum {
+  const float* vfreq;
+  int pair_half;
+  const T* gate;
+  int gate_stride;
+};
+__device__ __forceinline__ void turn_back(float& u, float& v, float pos, float freq) {
+  float sn, cs;
+  sincosf(__fmul_rn(pos, freq), &sn, &cs);
+  rotate_pair(u, v, cs, -sn, u, v);
+}
+template <typename T>
+__device__ __forceinline__ float gate_of(const AfterSum<T>& after, int tok, int head) {
+  return after.gate ? 1.0f / (1.0f + expf(-to_f32<T>(after.gate[(size_t)tok * after.gate_stride + head]))) : 1.f;
+}
+
 // SPLIT: the NW wavefronts of a workgroup share one tile and take its key steps in turn
 // (wavefront w the steps w, w + NW, ..); they add up through LDS, always in wavefront order.
 // For steps of few tiles (single decoded tokens), whose walks would else be one long chain each.
@@ -64,7 +85,7 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     const T* __restrict__ vcache, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
     const int* __restrict__ tile_row0, int nq, int nkv, int dk, int dv, int P, int window, float scale,
-    const float* __restrict__ sink, const float* __restrict__ score_bias, int gg, int chunk = 0,
+    const float* __restrict__ sink, const float* __restrict__ score_bias, int gg, AfterSum<T> after, int chunk = 0,
     float* __restrict__ part = nullptr) {
   extern __shared__ float merge[];  // SPLIT: [waves][16] maxima, [waves][16] sums, [waves - 1][VT][4][64] weighted values
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
@@ -324,12 +345,41 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   }
   if (!live) return;
   const float inv = sig ? 1.f : keep / l;
+#pragma unroll
+  for (int t = 0; t < VT; ++t) o[t] = o[t] * inv;
+  if (after.vfreq) {
+    const float fp = (float)pos;
+    if (after.pair_half) {  // dv == 16 VT: element 16 t + 4 c + i meets the one of block t + VT / 2
+#pragma unroll
+      for (int t = 0; t < VT / 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float u = o[t][i], v = o[t + VT / 2][i];
+          turn_back(u, v, fp, after.vfreq[16 * t + 4 * c + i]);
+          o[t][i] = u;
+          o[t + VT / 2][i] = v;
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < VT; ++t)
+        if (16 * t < dv) {
+#pragma unroll
+          for (int i = 0; i < 4; i += 2) {
+            float u = o[t][i], v = o[t][i + 1];
+            turn_back(u, v, fp, after.vfreq[(16 * t + 4 * c + i) / 2]);
+            o[t][i] = u;
+            o[t][i + 1] = v;
+          }
+        }
+    }
+  }
+  const float g = gate_of(after, tok, head);
   T* dst = out + (size_t)tok * out_stride + (size_t)head * dv;
 #pragma unroll
   for (int t = 0; t < VT; ++t) {
     if (16 * t < dv) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[t][i] * inv);
+      for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[t][i] * g);
     }
   }
 }
@@ -340,9 +390,10 @@ template <typename T, int VT>
 __global__ __launch_bounds__(VT * TK_WAVE) void attention_tile_merge_kernel(
     const float* __restrict__ part, int chunks, T* __restrict__ out, int out_stride, const int* __restrict__ q_start,
     const int* __restrict__ tile_req, const int* __restrict__ tile_row0, int nq, int nkv, int dv,
-    const float* __restrict__ sink, int gg, int plain_sums) {
+    const float* __restrict__ sink, int gg, int plain_sums, const int* __restrict__ kv_len, AfterSum<T> after) {
+  __shared__ float ex[VT * TK_WAVE * 4];  // the wavefronts' results, where the halves of a head are turned back
   const int lane = threadIdx.x & (TK_WAVE - 1), t = threadIdx.x / TK_WAVE;
-  if (16 * t >= dv) return;
+  if (16 * t >= dv) return;  // (never with halves to turn back: dv is 16 VT then, and every wavefront reaches the barrier)
   const int group = nq / nkv, blocks_per_kv = group / gg;
   const int hb = blockIdx.y, tile = blockIdx.x;
   const int head0 = (hb / blocks_per_kv) * group + (hb % blocks_per_kv) * gg;
@@ -375,11 +426,36 @@ __global__ __launch_bounds__(VT * TK_WAVE) void attention_tile_merge_kernel(
     keep = (m_all == -INFINITY) ? 0.f : expf(m_all - m2);
     l = l * keep + expf(sk - m2);
   }
+  const float inv = !live ? 0.f : (plain_sums ? 1.f : keep / l);  // (sigmoid weights: every chunk's maximum is 0 and its sums count as they are)
+  float r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = live ? o[i] * inv : 0.f;
+  if (after.vfreq) {
+    const int req = tile_req[tile];
+    const float fp = live ? (float)(kv_len[req] - (q_start[req + 1] - tok)) : 0.f;
+    if (after.pair_half) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ex[(t * TK_WAVE + lane) * 4 + i] = r[i];
+      __syncthreads();
+      const bool low = t < VT / 2;
+      const int other = low ? t + VT / 2 : t - VT / 2;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float u = low ? r[i] : ex[(other * TK_WAVE + lane) * 4 + i];
+        float v = low ? ex[(other * TK_WAVE + lane) * 4 + i] : r[i];
+        turn_back(u, v, fp, after.vfreq[16 * (low ? t : other) + 4 * c + i]);
+        r[i] = low ? u : v;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; i += 2) turn_back(r[i], r[i + 1], fp, after.vfreq[(16 * t + 4 * c + i) / 2]);
+    }
+  }
   if (!live) return;
-  const float inv = plain_sums ? 1.f : keep / l;  // (sigmoid weights: every chunk's maximum is 0 and its sums count as they are)
+  const float g = gate_of(after, tok, head);
   T* dst = out + (size_t)tok * out_stride + (size_t)head * dv;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[i] * inv);
+  for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(r[i] * g);
 }
 
 // Whether this kernel takes the shape (else the caller uses the plain 32-bit kernel).
@@ -387,6 +463,10 @@ TK_API int tk_attention_tile_f32_fits(int nq, int nkv, int dk, int dv, int P) {
   return (nq > 0 && nkv > 0 && nq % nkv == 0 && dk > 0 && dk % 8 == 0 && dk <= 32 * AT_MAX_KM && dv > 0 && dv % 16 == 0 &&
           dv <= 16 * AT_MAX_VT && P > 0 && P % 16 == 0) ? 1 : 0;
 }
+
+// Whether the kernel can turn back the halves of a value head of dv elements itself: the two elements of a pair lie in
+// one lane where the head fills the kernel's blocks of 16 (dv is 16 times 2, 4, 8 or 16).
+TK_API int tk_attention_tile_turns_halves(int dv) { return (dv == 32 || dv == 64 || dv == 128 || dv == 256) ? 1 : 0; }
 
 // 32-bit words of `part` that a (tile, head block, chunk) takes for a value head of dv elements
 TK_API int tk_attention_tile_part_words(int dv) {
@@ -400,27 +480,30 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
                       const void* kcache, const void* vcache, const int* block_table, int table_stride,
                       const int* q_start, const int* kv_len, const int* tile_req, const int* tile_row0, int nq,
                       int nkv, int dk, int dv, int P, int window, float scale, const float* sink, const float* score_bias,
-                      int gg, int chunk, float* part) {
+                      int gg, int chunk, float* part, const float* vfreq, int v_pair_half, const void* gate, int gate_stride) {
+  // halves of a head meet inside a lane only where the head fills the kernel's blocks of 16 (the entry point has checked)
+  const AfterSum<T> after = {vfreq, v_pair_half, (const T*)gate, gate_stride};
+  const AfterSum<T> none = {nullptr, 0, nullptr, 0};
   if (split && chunk > 0) {
     constexpr int NW = VT <= 4 ? 8 : 4;
     const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW, true>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
                        table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg,
-                       chunk, part);
+                       none, chunk, part);
     hipLaunchKernelGGL((attention_tile_merge_kernel<T, VT>), dim3(grid.x, grid.y), dim3(VT * TK_WAVE), 0, stream, part, (int)grid.z,
-                       (T*)out, out_stride, q_start, tile_req, tile_row0, nq, nkv, dv, sink, gg, score_bias ? 1 : 0);
+                       (T*)out, out_stride, q_start, tile_req, tile_row0, nq, nkv, dv, sink, gg, score_bias ? 1 : 0, kv_len, after);
   } else if (split) {
     // eight wavefronts a tile where their sums fit the local memory, else four
     constexpr int NW = VT <= 4 ? 8 : 4;
     const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
-                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg);
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, after);
   } else {
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, false, AT_WAVES>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
-                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg);
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, after);
   }
 }
 
@@ -431,7 +514,7 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
                                  const int* kv_len, const int* tile_req, const int* tile_row0, int n_tiles, int nq,
                                  int nkv, int dk, int dv, int P, int window, float scale, const float* sink,
                                  const float* score_bias, int gg, int split, int chunk, int chunks, float* part,
-                                 hipStream_t stream) {
+                                 const float* vfreq, int v_pair_half, const void* gate, int gate_stride, hipStream_t stream) {
   TK_REQUIRE(tk_attention_tile_f32_fits(nq, nkv, dk, dv, P), "attention_tile_f32: shape nq=%d nkv=%d dk=%d dv=%d P=%d not taken",
              nq, nkv, dk, dv, P);
   const int group = nq / nkv;
@@ -440,6 +523,9 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
   if (n_tiles <= 0) return 0;
   const int head_blocks = nkv * (group / gg);
   const int km = (dk + 31) / 32, vt = dv / 16;
+  TK_REQUIRE(!vfreq || (dv % 2 == 0 && (!v_pair_half || tk_attention_tile_turns_halves(dv))),
+             "attention_tile_f32: the halves of a value head of %d do not meet inside a lane", dv);
+  TK_REQUIRE(!gate || gate_stride >= nq, "attention_tile_f32: gate rows of %d hold no %d heads", gate_stride, nq);
   const bool sp = split != 0;
   const bool parts = sp && chunk > 0;
   TK_REQUIRE(!parts || (chunk % 128 == 0 && chunks > 0 && chunks < 65536 && part), "attention_tile_f32: chunks of a multiple of 128 keys, "
@@ -447,7 +533,8 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
   const dim3 grid(n_tiles, sp ? head_blocks : (head_blocks + AT_WAVES - 1) / AT_WAVES, parts ? chunks : 1);
   TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
 #define AT_ARGS grid, sp, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \
-                tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, parts ? chunk : 0, part
+                tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, parts ? chunk : 0, part, vfreq, v_pair_half, \
+                gate, gate_stride
 #define AT_VT(T, KMV)                                      \
   do {                                                     \
     if (vt <= 2) at_launch<T, KMV, 2>(AT_ARGS);            \

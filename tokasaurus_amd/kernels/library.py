@@ -57,7 +57,8 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_head_linear": [c_int, _P, c_int, _P, _P, c_int, c_int] + [c_int] * 4 + [_P],
         "tk_squared_relu": [c_int, _P, c_size_t, _P],
         "tk_attention_tile_f32": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P] + [c_int] * 7
-        + [c_float, _P, _P, c_int, c_int, c_int, c_int, _P, _P],
+        + [c_float, _P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, _P, c_int, _P],
+        "tk_attention_tile_turns_halves": [c_int],
         "tk_attention_tile_part_words": [c_int],
         "tk_attention_tile_f32_fits": [c_int] * 5,
         "tk_delta_prepare": [c_int, _P, c_int, c_int, _P, c_int, _P, c_int, _P, _P, _P, c_size_t, c_size_t, _P, _P, _P, _P]

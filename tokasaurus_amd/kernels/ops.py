@@ -1372,6 +1372,11 @@ def attention_tile_f32_fits(nq: int, nkv: int, key_dim: int, value_dim: int, pag
     return bool(load("core").tk_attention_tile_f32_fits(nq, nkv, key_dim, value_dim, page_size))
 
 
+def attention_tile_turns_halves(value_dim: int) -> bool:
+    """Whether the matrix-core attention can itself turn back the halves of a value head of this size."""
+    return bool(load("core").tk_attention_tile_turns_halves(int(value_dim)))
+
+
 ATTENTION_TILE_SPLIT_BELOW = 2048  # (tile, head block) pairs of a step below which the wavefronts share tiles
 ATTENTION_TILE_WORKGROUPS = 512  # workgroups a step with key chunks should have before its chunks grow
 ATTENTION_TILE_LONGEST_CHUNK = 2048
@@ -1394,7 +1399,8 @@ def attention_tile_f32(
     kv_len: torch.Tensor, tile_req: torch.Tensor, tile_row0: torch.Tensor, nq: int, nkv: int, key_dim: int,
     value_dim: int, page_size: int, heads_a_tile: int, window: int = 0, scale: float = 1.0,
     sink: torch.Tensor | None = None, split: bool | None = None, key_chunk: int = 0, longest: int = 0, first_row: int = 0,
-    score_bias: torch.Tensor | None = None,
+    score_bias: torch.Tensor | None = None, value_freq: torch.Tensor | None = None,
+    value_pair_halves: bool = False, gate: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Attention in 32-bit arithmetic on the matrix cores: every token of the step over its
     request's pages; ``tile_req`` / ``tile_row0`` name each tile's request and its first token's
@@ -1406,8 +1412,15 @@ def attention_tile_f32(
     depend on the batch): a split tile's keys are also cut at absolute multiples of ``key_chunk`` among
     workgroups, whose partial results a second kernel adds in ascending order.
     ``first_row``: ``q`` holds the step's rows from this one on only (the tiles name none before it), and so
-    does the result.  ``score_bias``: sigmoid weights as in ``paged_attention_generic``."""
-    _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink, score_bias)
+    does the result.  ``score_bias``: sigmoid weights as in ``paged_attention_generic``.  ``value_freq``,
+    ``value_pair_halves``, ``gate``: what ``unrotate_gate_`` does, in the kernel's own epilogue (halves only where
+    ``attention_tile_turns_halves``)."""
+    _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink, score_bias, value_freq, gate)
+    _f32_vector(value_freq, value_dim // 2, "attention: the values' frequencies")
+    _need(value_freq is None or not value_pair_halves or attention_tile_turns_halves(value_dim),
+          "attention: the halves of this value size are turned back by unrotate_gate_")
+    _need(gate is None or (gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[1] == nq and gate.dtype == q.dtype
+                           and gate.shape[0] == q.shape[0]), "attention: one gate a token and head, of the rows' type")
     _f32_vector(score_bias, nq, "attention: the scores' biases")
     if split is None:
         split = tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) < ATTENTION_TILE_SPLIT_BELOW
@@ -1445,7 +1458,10 @@ def attention_tile_f32(
          kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(), tile_req.numel(), nq, nkv, key_dim, value_dim,
          page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None,
          score_bias.data_ptr() if score_bias is not None else None, int(heads_a_tile),
-         1 if split else 0, int(key_chunk) if chunks else 0, chunks, part.data_ptr() if part is not None else None, _stream())
+         1 if split else 0, int(key_chunk) if chunks else 0, chunks, part.data_ptr() if part is not None else None,
+         value_freq.data_ptr() if value_freq is not None else None, 1 if value_pair_halves else 0,
+         (gate.data_ptr() - int(first_row) * gate.stride(0) * gate.element_size()) if gate is not None else None,
+         gate.stride(0) if gate is not None else 0, _stream())
     return out
 
 

@@ -224,20 +224,26 @@ class GroupedAttention(Mixer):
                        values_are_keys=self.values_are_keys, per_head=self.head_norm is not None,
                        value_freq=self.value_freq, value_pair_halves=v_halves,
                        rotation_scale=self.position.magnitude if self.position is not None else 1.0)
+        gate = qkv[:, self.gate_col : self.gate_col + nq] if self.gate_col is not None else None
+        after = self.value_freq is not None or gate is not None
         if ops.attention_tile_f32_fits(nq, nkv, dk, dv, cache.page_size):
+            # the kernel turns the heads' results back and gates them itself where the pairs lie inside its lanes
+            fused = after and (self.value_freq is None or not v_halves or ops.attention_tile_turns_halves(dv))
             gg = ops.attention_tile_heads(nq // nkv, ctx.max_q_len)
             tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
             attn = ops.attention_tile_f32(qkv, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
                                           tile_req, tile_row0, nq, nkv, dk, dv, cache.page_size, gg,
                                           window=self.window, scale=self.scale, sink=self.sink, key_chunk=self.key_chunk,
-                                          longest=ctx.extras.get("kv_bound", ctx.max_kv_len), score_bias=self.score_bias)
+                                          longest=ctx.extras.get("kv_bound", ctx.max_kv_len), score_bias=self.score_bias,
+                                          value_freq=self.value_freq if fused else None, value_pair_halves=v_halves,
+                                          gate=gate if fused else None)
+            after = after and not fused
         else:  # sizes that the matrix-core kernel does not take
             attn = ops.paged_attention_generic(qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
                                                nq, nkv, dk, cache.page_size, window=self.window, scale=self.scale,
                                                value_dim=dv, sink=self.sink, score_bias=self.score_bias)
-        if self.value_freq is not None or self.gate_col is not None:
+        if after:
             # the heads' results turned back by their own positions, then each head's gate
-            gate = qkv[:, self.gate_col : self.gate_col + nq] if self.gate_col is not None else None
             ops.unrotate_gate_(attn, ctx.positions, self.value_freq, v_halves, gate, nq, dv)
         return attn if rows is None else ops.gather_rows(attn, rows)
 
