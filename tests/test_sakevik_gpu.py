@@ -315,6 +315,41 @@ def test_long_decoding(sakevik_folders, dtype):
     assert all(step.captured for step in runner.recorded.values()) and runner.recorded
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_requests_across_context_bounds(tmp_path, dtype):
+    """Requests of up to 2 100 tokens: steps planned for 1 024, 2 048 and 4 096 tokens of context, windows shorter and
+    longer than a chunk of keys and none, portions of hundreds of tokens after pasts of which a windowed cache has given
+    most pages back, 500 tokens decoded one by one, and three requests of unequal length in one batch."""
+    config = model(210, 96, [
+        attention_layer(4, 2, 32, 32, 0.18, 16, 3000.0, window=180, mlp=dense(128, 2.0)),
+        latent_layer(4, 32, 16, 32, 80, 0.14, 1e6, window=520, scaling={"factor": 4.0, "original": 256, "fast": 16.0, "slow": 1.0},
+                     mlp=dense(128, 3.0)),
+        gru_layer(160),
+        latent_layer(2, 16, 8, 16, 40, 0.2, 1e4, mlp=dense(64, 2.0)),
+        attention_layer(3, 3, 16, 64, 0.25, 16, 1e4, window=1300),
+    ], scale=9.0, logit_scale=1.5, bigram=(211, 13, 5))
+    folder = make_folder(tmp_path / "long", config, seed=3)
+    n = 2100
+    reqs = {"a": random_tokens(n, 210, 1), "b": random_tokens(600, 210, 2), "c": random_tokens(1200, 210, 3)}
+    plain = plain_rows(folder, reqs)
+    runner = runner_for(folder, dtype, tokens=4096)
+
+    def some(got, every=9):
+        return {k: v for i, (k, v) in enumerate(sorted(got.items())) if i % every == 0 or k[1] > n - 40}
+
+    tol = TOL[dtype]
+    compare_rows(some(run_steps(runner, whole("a", reqs["a"]))), plain, tol)
+    compare_rows(some(run_steps(runner, portions("a", reqs["a"], [512, 3, 700, 64, 2, 600]))), plain, tol)
+    compare_rows(some(run_steps(runner, tail_one_by_one("a", reqs["a"], tail=500))), plain, tol)
+    a, b, c = reqs["a"], reqs["b"], reqs["c"]
+    steps = [{"entries": [("a", a[:1000], [999]), ("b", b[:300], [0, 299])]},
+             {"entries": [("a", a[1000:2000], [0, 999]), ("b", b[300:301], [0]), ("c", c[:1100], [1099])]},
+             {"entries": [("a", a[2000:2001], [0]), ("b", b[301:600], [298]), ("c", c[1100:1101], [0])], "end": ["b"]},
+             {"entries": [("a", a[2001:], [n - 2002]), ("c", c[1101:], [98])], "end": ["a", "c"]}]
+    compare_rows(run_steps(runner, steps), plain, tol)
+    assert runner.manager.requests == {}
+
+
 @pytest.mark.parametrize("name", ["mixed", "awkward", "only_gru"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_engine(sakevik_folders, dtype, name):
