@@ -403,7 +403,7 @@ def sakevik_like(size: dict, layers: int) -> dict:
         "rot": {"base": ll["rope_theta"], "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}}
     gru = {"type": "mingru", "mlp": None, "mixer": {"width": 2 * ll["hidden_size"]}}
     return {"architecture": "Sakevik", "vocab": ll["vocab_size"], "width": ll["hidden_size"], "norm": {"eps": 1e-6},
-            "embedding": {"scale": float(ll["hidden_size"]) ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "embedding": {"scale": float(ll["hidden_size"]) ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 1009, "mul_cur": 917}},
             "logit_scale": 0.5, "layers": [(attention, latent, gru, attention)[i % 4] for i in range(layers)]}
 
 

@@ -451,7 +451,7 @@ def random_config(seed: int) -> dict:
             layers.append(latent_layer(rng.choice([1, 2, 3, 8]), rng.choice([8, 12, 16, 32]), rot_dim, rng.choice([4, 8, 16, 24]),
                                        rng.choice([8, 17, 32, 64, 96]), rng.choice([0.1, 0.3]), rng.choice([10.0, 1e4, 1e6]),
                                        window=window, scaling=scaling, rot_dims=rng.choice([rot_dim, 2]), mlp=mlp))
-    bigram = rng.choice([None, (rng.choice([1, 2, 61, 509]), rng.choice([1, 31, 12345]), rng.choice([1, 7, 999]))])
+    bigram = rng.choice([None, (rng.choice([1, 2, 61, 499]), rng.choice([1, 29, 12345]), rng.choice([1, 11, 999]))])
     return model(rng.choice([40, 97, 130]), width, layers, eps=rng.choice([1e-6, 1e-5]), scale=rng.choice([1.0, 6.0]),
                  bigram=bigram, logit_scale=rng.choice([None, 0.25, 3.0]))
 
