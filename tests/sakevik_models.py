@@ -21,8 +21,10 @@ import plain_sakevik
 from tokasaurus_amd.weights import write_random_model
 
 
-def attention_layer(heads, kv_heads, dim, vdim, scale, rot_dims, base, window=None, mlp=None):
+def attention_layer(heads, kv_heads, dim, vdim, scale, rot_dims, base, window=None, mlp=None, scaling=None):
     mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "rot": {"base": base, "dims": rot_dims}}
+    if scaling is not None:
+        mixer["rot"]["scaling"] = scaling
     if window is not None:
         mixer["mask"] = {"size": window}
     return {"type": "attention", "mixer": mixer, "mlp": mlp}

@@ -68,7 +68,7 @@ def test_recurrence_kernel(width, lens):
     state = state0.clone()
     bias = torch.randn(2 * width, device=dev)
     out = ops.min_gru(proj, state, q_start, slots, width, max(lens), torch.float32, bias=bias)
-    p = proj.double().cpu()
+    p = proj.double().cpu().view(n, width, 3).permute(0, 2, 1).reshape(n, 3 * width)  # (a, u, g) a channel -> [a | u | g]
     p[:, : 2 * width] += bias.double().cpu()
     for r, l in enumerate(lens):
         S = state0[int(slots[r])].double().cpu()
@@ -147,6 +147,7 @@ SINGLE_LAYERS = {
     "attention_sizes_off_every_multiple": attention_layer(3, 1, 12, 6, 0.3, 6, 50.0, window=5),
     "attention_heads_of_128": attention_layer(4, 2, 128, 128, 0.09, 64, 500000.0, window=30),
     "attention_values_of_48": attention_layer(2, 1, 64, 48, 0.12, 32, 10000.0, window=25),
+    "attention_with_ramp_on_queries_and_keys": attention_layer(4, 2, 32, 32, 0.2, 16, 500.0, window=40, scaling=RAMP),
     "latent_with_ramp": latent_layer(3, 24, 8, 40, 48, 0.2, 1000.0, window=30, scaling=RAMP),
     "latent_no_ramp_no_window": latent_layer(2, 16, 16, 16, 32, 0.25, 100.0),
     "latent_part_of_the_rotated_part_turned": latent_layer(4, 8, 8, 8, 24, 0.3, 20.0, window=12, rot_dims=4),

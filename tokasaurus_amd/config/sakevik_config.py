@@ -9,7 +9,7 @@ two models of the design is taken from it.  Keys:
     layers[i].mlp: null | {"kind": "dense", "ff": n, "limit": x}
     mingru mixer:           width
     attention mixer:        heads, kv_heads, dim, vdim, scale, mask: absent or null | {size},
-                            rot: {base, dims}
+                            rot: {base, dims, scaling: absent or null | as below (queries and keys only)}
     latent_attention mixer: heads, dim, rot_dim, vdim, kv_rank, scale, mask: absent or null | {size},
                             rot: {base, dims, scaling: absent or null | {factor, original, fast, slow}}
 """

@@ -1,8 +1,10 @@
 // A gated recurrence whose gates read the current token only (minGRU): per channel
 //     z = sigmoid(a + b_z),   u' = u + b_x,   cand = u' + 1/2 where u' >= 0, sigmoid(u') where u' < 0,
 //     S_t = (1 - z) S_(t-1) + z cand,     out_t = S_t * silu(g)
-// on the 32-bit sums [a | u | g] of one stacked product; the two biases (32-bit, [2 width], or null) are
-// added here, which saves the product a pass over its result.  The state S is one 32-bit number a
+// on the 32-bit sums of one stacked product whose rows are interleaved channel by channel, (a, u, g) of channel 0,
+// then of channel 1, ..: a lane reads its channel's three sums as 12 neighbouring bytes and a wavefront 768 of a
+// token's row (with [a | u | g] it read three pieces of 256 bytes thousands of bytes apart).  The two biases
+// (32-bit, [b_z | b_x], or null) are added here, which saves the product a pass over its result.  The state S is one 32-bit number a
 // channel in the request's slot; a step of any cut continues from it.  Everything is 32-bit
 // arithmetic; `out` is rounded once to the storage type.
 //
@@ -36,8 +38,8 @@ __global__ __launch_bounds__(W * TK_WAVE) void min_gru_kernel(const float* __res
 #pragma unroll
     for (int i = 0; i < L; ++i) {
       const bool in = live && t0 + i < end;
-      const float* src = proj + (size_t)(in ? t0 + i : first) * stride + (live ? ch : 0);
-      const float a = src[0] + bz, u = src[width] + bx, g = src[2 * width];
+      const float* src = proj + (size_t)(in ? t0 + i : first) * stride + 3 * (live ? ch : 0);
+      const float a = src[0] + bz, u = src[1] + bx, g = src[2];
       const float z = 1.0f / (1.0f + expf(-a));
       const float cand = u >= 0.f ? u + 0.5f : 1.0f / (1.0f + expf(-u));
       keep[i] = 1.0f - z;

@@ -1232,13 +1232,13 @@ def min_gru(proj: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, slot
             out_dtype: torch.dtype, bias: torch.Tensor | None = None) -> torch.Tensor:
     """The gated recurrence ``S <- (1 - z) S + z cand`` per channel over every request's tokens of this
     step, from and to the request's slot of ``state`` [slots, width] (32-bit): ``proj`` holds the 32-bit
-    sums [a | u | g] ([tokens, 3 width]; z = sigmoid(a), cand = u + 1/2 for u >= 0 and sigmoid(u) below);
+    sums (a, u, g) channel by channel ([tokens, width * 3]; z = sigmoid(a), cand = u + 1/2 for u >= 0 and sigmoid(u) below);
     returns S_t * silu(g) rounded once to ``out_dtype``.  ``longest``: the most tokens a request brings.
     ``bias`` (32-bit, [2 width]): added to a and to u here, when the product has not."""
     _gpu(proj, state, q_start, slots, bias)
     _f32_vector(bias, 2 * width, "min_gru: the biases of z and of the candidate")
     _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1 and proj.shape[1] >= 3 * width,
-          "min_gru: 32-bit rows [a | u | g]")
+          "min_gru: 32-bit rows of (a, u, g) a channel")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.stride(1) == 1 and state.shape[1] >= width,
           "min_gru: the state is 32-bit [slots, width]")
     _i32(q_start, "q_start")

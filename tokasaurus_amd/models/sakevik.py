@@ -24,6 +24,9 @@ def sakevik_spec(cfg: SakevikConfig) -> ModelSpec:
     def norm(name: str) -> PartSpec:
         return PartSpec("stream_rmsnorm", {"size": cfg.width, "eps": cfg.norm_eps, "name": name})
 
+    def ramp_of(rot) -> dict | None:
+        return dict(zip(("factor", "original", "fast", "slow"), rot.scaling)) if rot.scaling is not None else None
+
     layers, unused = [], []
     for i, layer in enumerate(cfg.layers):
         m, p = layer.mixer, f"l{i}.mix"
@@ -35,7 +38,9 @@ def sakevik_spec(cfg: SakevikConfig) -> ModelSpec:
             mixer = PartSpec("grouped_attention", {
                 "hidden_size": cfg.width, "num_heads": m.heads, "num_kv_heads": m.kv_heads, "key_dim": m.dim, "value_dim": m.vdim,
                 "scale": m.scale, "window": m.window, "key_chunk": 256,
-                "position": PartSpec("rotary_halves", {"dims": m.rot.dims, "base": m.rot.base}),
+                # (a ramp between frequency scales, where the file gives one, is the queries' and keys' alone: the values turn
+                # by the plain frequencies of the same base)
+                "position": PartSpec("rotary_halves", {"dims": m.rot.dims, "base": m.rot.base, "ramp": ramp_of(m.rot)}),
                 "names": {"q": f"{p}.q", "k": f"{p}.k", "v": f"{p}.v", "o": f"{p}.o"},
                 "bias_names": {"q": f"{p}.q.b", "k": f"{p}.k.b", "v": f"{p}.v.b", "o": f"{p}.o.b"},
                 "head_norm": {"q": f"{p}.q.norm", "k": f"{p}.k.norm", "eps": cfg.norm_eps},
@@ -44,13 +49,10 @@ def sakevik_spec(cfg: SakevikConfig) -> ModelSpec:
                 "gate_name": f"{p}.g"})
         else:
             assert isinstance(m, RotatedLatentAttentionLayer)
-            ramp = None
-            if m.rot.scaling is not None:
-                ramp = dict(zip(("factor", "original", "fast", "slow"), m.rot.scaling))
             mixer = PartSpec("latent_attention", {
                 "hidden_size": cfg.width, "num_heads": m.heads, "key_dim": m.dim, "value_dim": m.vdim, "q_rank": 0,
                 "kv_rank": m.kv_rank, "rot_dim": m.rot_dim, "scale": m.scale, "norm_eps": cfg.norm_eps, "window": m.window,
-                "position": PartSpec("rotary_interleaved", {"dims": m.rot.dims, "base": m.rot.base, "ramp": ramp}),
+                "position": PartSpec("rotary_interleaved", {"dims": m.rot.dims, "base": m.rot.base, "ramp": ramp_of(m.rot)}),
                 "names": {"q": f"{p}.q", "dkv": f"{p}.dkv", "dkv_norm": f"{p}.dkv.norm", "uk": f"{p}.uk", "uv": f"{p}.uv",
                           "o": f"{p}.o"}})
         params = {"mixer": mixer, "mixer_post_norm": norm(f"l{i}.norm1")}

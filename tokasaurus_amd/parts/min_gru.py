@@ -3,7 +3,8 @@ request, one number a channel instead of keys and values.
 
 Per token and channel: ``z = sigmoid(W_z h + b_z)``, ``u = W_x h + b_x``, the candidate
 ``c = u + 1/2`` where ``u >= 0`` and ``sigmoid(u)`` below; ``S <- (1 - z) S + z c``; the output is
-``W_o (S * silu(W_g h))``.  z, x and g are one stacked product whose 32-bit sums (biases added) go
+``W_o (S * silu(W_g h))``.  z, x and g are one stacked product (its rows interleaved channel by channel,
+so that the recurrence reads a channel's three sums side by side) whose 32-bit sums go
 straight into the recurrence, whose kernel adds the two biases: gates, candidate and state are 32-bit
 arithmetic in either storage type.  The state is one row of 32-bit numbers in the request's slot, zero when a request takes the
 slot; a step of any cut continues from it with the same bits as the token-by-token recurrence.
@@ -36,7 +37,13 @@ class MinGRU(Mixer):
         return StateNeed((self.width,), torch.float32)
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
-        self.inp.load(tensors, placer)
+        z, x, g = self.inp.names
+
+        def interleaved() -> torch.Tensor:  # rows (z_c, x_c, g_c) for channel c = 0, 1, ..
+            w = torch.stack([tensors[z], tensors[x], tensors[g]], dim=1)
+            return w.reshape(3 * self.width, self.hidden_size).to(dtype=placer.dtype).contiguous().to(placer.device)
+
+        self.inp.weight = placer.place(("rows_interleaved", z, x, g), interleaved)
         self.out.load(tensors, placer)
         self.bias = placer.place(("vector_f32", *self.bias_names), lambda: torch.cat(
             [tensors[b].to(torch.float32) for b in self.bias_names]).contiguous().to(placer.device))
