@@ -10,12 +10,19 @@
 //
 // A workgroup owns 64 neighbouring channels of one request (a lane a channel, so a wavefront's
 // loads are whole lines).  The chain S_t is the only thing that is sequential: the W wavefronts of a
-// workgroup each take L neighbouring tokens of a round of W * L, load them and compute gates and
+// workgroup each take L neighbouring tokens of a round of W * L, load them (a round ahead) and compute gates and
 // candidates side by side, and then the state passes through the wavefronts in order, L
 // multiply-adds each and nothing else (the products with the gates and the stores follow when the
 // state has moved on).  The sums are those of the plain recurrence token by token, whatever the cut
 // of the prompt and whatever W: the same bits.
 #include "common.h"
+
+// 1 / (1 + exp(-x)) on the hardware's own exponential and reciprocal (an instruction each, an ulp each): three of
+// these a token and channel are most of this kernel's arithmetic, and with the library's exponential and an exact
+// division they, not the chain or the bytes, set its time (exp2(inf) = inf gives 1 / inf = 0, exp2(-inf) = 0 gives 1).
+__device__ __forceinline__ float sigmoid_hw(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + exp2f(x * -1.44269504088896341f));
+}
 
 template <typename T, int W, int L>
 __global__ __launch_bounds__(W * TK_WAVE) void min_gru_kernel(const float* __restrict__ proj, int stride, const float* __restrict__ bias,
@@ -32,20 +39,33 @@ __global__ __launch_bounds__(W * TK_WAVE) void min_gru_kernel(const float* __res
   const float bz = bias && live ? bias[ch] : 0.f, bx = bias && live ? bias[width + ch] : 0.f;
   if (wave == 0) carry[lane] = live ? *sp : 0.f;
   if (W > 1) __syncthreads();
+  // a round's sums are asked for while the round before still hands the state on
+  float ra[L], ru[L], rg[L];
+  auto ask = [&](int base) {
+    const int t0 = base + wave * L;
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+      const bool in = live && t0 + i < end;
+      const float* src = proj + (size_t)(in ? t0 + i : first) * stride + 3 * (live ? ch : 0);
+      ra[i] = src[0];
+      ru[i] = src[1];
+      rg[i] = src[2];
+    }
+  };
+  ask(first);
   for (int base = first; base < end; base += W * L) {
     const int t0 = base + wave * L;
     float keep[L], add[L], gate[L];
 #pragma unroll
     for (int i = 0; i < L; ++i) {
-      const bool in = live && t0 + i < end;
-      const float* src = proj + (size_t)(in ? t0 + i : first) * stride + 3 * (live ? ch : 0);
-      const float a = src[0] + bz, u = src[1] + bx, g = src[2];
-      const float z = 1.0f / (1.0f + expf(-a));
-      const float cand = u >= 0.f ? u + 0.5f : 1.0f / (1.0f + expf(-u));
+      const float a = ra[i] + bz, u = ru[i] + bx, g = rg[i];
+      const float z = sigmoid_hw(a);
+      const float cand = u >= 0.f ? u + 0.5f : sigmoid_hw(u);
       keep[i] = 1.0f - z;
       add[i] = z * cand;
-      gate[i] = g / (1.0f + expf(-g));
+      gate[i] = g * sigmoid_hw(g);
     }
+    if (base + W * L < end) ask(base + W * L);
 #pragma unroll 1
     for (int phase = 0; phase < W; ++phase) {
       if (wave == phase && t0 < end) {
@@ -82,7 +102,7 @@ TK_API int tk_min_gru(int dt, const float* proj, int stride, const float* bias, 
   } else if (longest <= 64) {
     if (dt == TK_F32) MG_LAUNCH(float, 4, 16); else MG_LAUNCH(bf16_t, 4, 16);
   } else {
-    if (dt == TK_F32) MG_LAUNCH(float, 16, 16); else MG_LAUNCH(bf16_t, 16, 16);
+    if (dt == TK_F32) MG_LAUNCH(float, 8, 16); else MG_LAUNCH(bf16_t, 8, 16);
   }
 #undef MG_LAUNCH
   TK_CHECK_LAUNCH("min_gru");
