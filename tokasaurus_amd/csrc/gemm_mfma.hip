@@ -75,6 +75,7 @@ struct GemmArgs {
   // the gated epilogue's other form (glu_limit > 0): g = min(gate, limit), u = clamp(up, -limit, limit),
   // g * sigmoid(glu_alpha * g) * (u + 1), 32-bit until the one rounding at the store
   float glu_limit, glu_alpha;
+  float out_scale;  // the 32-bit epilogue multiplies its result by this (1: as it is)
   int M, N, K;  // N: outputs (for SwiGLU the intermediate size; W then has 2N rows, gate first)
   int TH;       // weight rows of a tile that are used (16, or 8 to make twice the workgroups of a narrow output)
 };
@@ -106,6 +107,8 @@ __device__ __forceinline__ void store4(const GemmArgs& a, f32x4_t v, f32x4_t up,
       o[j] = round_to<bf16_t>(o[j]) + __bfloat162float(a.residual[(size_t)token * a.ldr + n + j]);
   }
   if (EPI == EPI_F32) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] *= a.out_scale;
     float* c = (float*)a.C + (size_t)token * a.ldc + n;
     if (n + 3 < a.N && (a.ldc & 3) == 0) {
       *(f32x4_t*)c = f32x4_t{o[0], o[1], o[2], o[3]};
@@ -687,6 +690,8 @@ struct GemmExtra {
   const void* bias;
   // the gated epilogue with clamps (see GemmArgs); 0: the plain one
   float glu_limit, glu_alpha;
+  // a factor on the 32-bit epilogue's result; 0 stands for none
+  float out_scale;
 };
 
 // Number of partial sums a row gets from the residual epilogue with emit_w: one a tile.
@@ -754,6 +759,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
   GemmArgs a = {};
   a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.C = C; a.ldc = ldc;
   a.residual = (const bf16_t*)residual; a.ldr = ldr; a.M = M; a.N = N; a.K = K; a.TH = 16;
+  a.out_scale = 1.f;
   bool norm = false;
   if (extra) {
     a.sumsq_in = extra->sumsq_in; a.parts_in = extra->parts_in; a.eps = extra->eps;
@@ -765,6 +771,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
     a.nq = extra->nq; a.nkv = extra->nkv; a.d = extra->d; a.P = extra->P;
     a.bias = (const bf16_t*)extra->bias;
     a.glu_limit = extra->glu_limit; a.glu_alpha = extra->glu_alpha;
+    if (extra->out_scale != 0.f) a.out_scale = extra->out_scale;
     norm = a.sumsq_in != nullptr;
   }
   TK_REQUIRE(!norm || a.parts_in > 0, "gemm_skinny: a norm in front needs its partial sums");

@@ -839,6 +839,7 @@ class _GemmExtra(ctypes.Structure):
         ("kcache", ctypes.c_void_p), ("vcache", ctypes.c_void_p),
         ("nq", ctypes.c_int), ("nkv", ctypes.c_int), ("d", ctypes.c_int), ("P", ctypes.c_int),
         ("bias", ctypes.c_void_p), ("glu_limit", ctypes.c_float), ("glu_alpha", ctypes.c_float),
+        ("out_scale", ctypes.c_float),
     ]
 
 
@@ -887,6 +888,7 @@ def gemm_skinny_bf16(
     bias: torch.Tensor | None = None,
     fold: bool = True,
     glu: tuple[float, float] | None = None,
+    out_scale: float | None = None,
 ):
     """a [M <= 128, K] times w [N, K] transposed on the matrix cores, with the
     epilogue fused: + residual, 32-bit output, (``swiglu``: w is [gate | up]
@@ -900,6 +902,7 @@ def gemm_skinny_bf16(
     ``bias`` (one value a row of ``w``): added to the product before the epilogue.
     ``glu`` (with ``swiglu``): (limit, alpha); the gated epilogue is then min(gate, limit) *
     sigmoid(alpha * min(gate, limit)) * (clamp(up, -limit, limit) + 1).
+    ``out_scale`` (with ``out_f32``): the 32-bit result is multiplied by it.
     ``waves_k``, ``tiles``, ``staged``, ``tile_rows``, ``fold``: the kernel's own choices overridden (for measurements)."""
     _gpu(a, w, residual, emit_weight, bias)
     _check_bias(bias, w, "gemm_skinny")
@@ -956,6 +959,10 @@ def gemm_skinny_bf16(
         epi = EPI_F32 if out_f32 else EPI_STORE
     if bias is not None:
         extra.bias = bias.data_ptr()
+        use_extra = True
+    if out_scale is not None and float(out_scale) != 1.0:
+        _need(epi == EPI_F32 and float(out_scale) != 0.0, "gemm_skinny: a factor on the result goes with 32-bit output and is not 0")
+        extra.out_scale = float(out_scale)
         use_extra = True
     if prenorm is not None:
         _gpu(prenorm.scaled, prenorm.sumsq)

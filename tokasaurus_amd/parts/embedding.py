@@ -119,7 +119,5 @@ class LMHead(Head):
     takes_out = True
 
     def forward(self, x: torch.Tensor, prepared: Prepared | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
-        logits = self.proj(Normed(x, self.norm, prepared), out_f32=True, out=out)
-        if self.scale is not None:
-            logits = ops.scale_(logits, self.scale)
+        logits = self.proj(Normed(x, self.norm, prepared), out_f32=True, out=out, out_scale=self.scale)
         return ops.softcap_(logits, self.softcap) if self.softcap is not None else logits

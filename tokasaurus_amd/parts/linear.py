@@ -100,6 +100,7 @@ class Linear:
         swiglu: bool = False,
         out: torch.Tensor | None = None,
         glu: tuple[float, float] | None = None,
+        out_scale: float | None = None,
     ) -> torch.Tensor:
         """x [M, in] -> [M, out].  ``residual``: returns residual + product (the
         product rounded to the storage type first).  ``out_f32``: 32-bit output.
@@ -108,7 +109,11 @@ class Linear:
         weight (a mixer that only needs its queries).  ``x`` may be a ``Normed``:
         the norm is folded into the product when it was prepared, else applied first.
         ``out`` (with ``out_f32``): a buffer [M, out] for the result, in place of new memory.
-        ``glu`` (with ``swiglu``): (limit, alpha) of the gated activation with clamps, in place of silu(gate) * up."""
+        ``glu`` (with ``swiglu``): (limit, alpha) of the gated activation with clamps, in place of silu(gate) * up.
+        ``out_scale`` (with ``out_f32``): the 32-bit result times this factor (in the few-row product's epilogue, else by a
+        pass of its own)."""
+        assert out_scale is None or (out_f32 and residual is None), "a factor on the result goes with 32-bit output"
+        scaled = (lambda p: ops.scale_(p, out_scale)) if out_scale is not None and float(out_scale) != 1.0 else (lambda p: p)
         gated = (lambda p: ops.clamped_glu(p, glu[0], glu[1])) if glu is not None else ops.swiglu
         assert out is None or (out_f32 and residual is None and not swiglu), "a result buffer goes with 32-bit output only"
         w, bias = self.weight, self.bias
@@ -126,7 +131,8 @@ class Linear:
         if w.dtype == torch.bfloat16 and m > 0 and (m > ops.SKINNY_ROWS or self._aligned()):
             if self._fast(m, swiglu, out_f32):
                 return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu,
-                                            prenorm=prenorm, norm_eps=eps, out=out, bias=bias, glu=glu if swiglu else None)
+                                            prenorm=prenorm, norm_eps=eps, out=out, bias=bias, glu=glu if swiglu else None,
+                                            out_scale=out_scale)
             # library matrix product (hipBLASLt), 32-bit accumulation; with a bias through the tensor
             # library, whose call adds it to the 32-bit sums in the product's own epilogue (addmm)
             direct = ops.gemm_library_direct(x, w)
@@ -136,7 +142,7 @@ class Linear:
                 else:
                     prod = (torch.mm(x, w.t(), out_dtype=torch.float32, out=out) if out is not None
                             else torch.mm(x, w.t(), out_dtype=torch.float32))
-                return ops.add_bias(prod, bias) if bias is not None else prod
+                return scaled(ops.add_bias(prod, bias) if bias is not None else prod)
             if bias is not None:
                 prod = torch.addmm(bias, x, w.t())
             else:
@@ -148,7 +154,7 @@ class Linear:
             return gated(prod) if swiglu else prod
         # the 32-bit path, and few bfloat16 rows of a width the matrix-core kernel does not take
         prod = ops.gemm_generic(x, w, residual=residual, out_f32=out_f32, out=out, bias=bias)
-        return gated(prod) if swiglu else prod
+        return gated(prod) if swiglu else scaled(prod)
 
     def with_residual(
         self, x: torch.Tensor, residual: torch.Tensor, emit_norm: Norm | None
