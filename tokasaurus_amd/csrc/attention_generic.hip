@@ -15,6 +15,8 @@
 // 32-bit number a query head): exp(sink) is added once to the softmax's denominator; it has no
 // key and no value.  `score_bias` (null, or one 32-bit number a query head): the weights are no
 // softmax but sigmoid(score + score_bias[head]) for every key the query sees, not normalised.
+// `softcap` (> 0): a scaled score becomes softcap * tanh(score / softcap).  `rel` (null, or [buckets][nq]):
+// rel[bucket_of[min(distance, far)]][head] is added to the score of a key `distance` positions back.
 #include "common.h"
 
 #define AG_THREADS 256
@@ -26,7 +28,8 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
     const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_req,
     const int* __restrict__ positions, int nq, int nkv, int d, int dv, int P, int window, float scale,
-    const float* __restrict__ sink, const float* __restrict__ score_bias) {
+    const float* __restrict__ sink, const float* __restrict__ score_bias, float softcap,
+    const int* __restrict__ bucket_of, int far, const float* __restrict__ rel) {
   extern __shared__ float smem[];
   const int t = blockIdx.x, g = blockIdx.y;
   const int group = nq / nkv;
@@ -86,6 +89,8 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
         const float* kv = Ks + j * (d + 1);
         for (int e = 0; e < d; ++e) dot = fmaf(qv[e], kv[e], dot);
         s = dot * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        if (rel) s += rel[(size_t)bucket_of[min(pos - kp, far)] * nq + g * group + gq];
       }
       Ss[i] = s;
     }
@@ -154,11 +159,12 @@ static void ag_launch(const void* q, int q_stride, void* out, int out_stride, co
                       const void* vcache, const int* block_table, int table_stride,
                       const int* token_req, const int* positions, int n_tokens, int nq, int nkv,
                       int d, int dv, int P, int window, float scale, const float* sink, const float* score_bias,
-                      hipStream_t stream) {
+                      float softcap, const int* bucket_of, int far, const float* rel, hipStream_t stream) {
   hipLaunchKernelGGL((paged_attention_generic_kernel<T, CH>), dim3(n_tokens, nkv),
                      dim3(AG_THREADS), ag_smem_bytes(nq / nkv, d, dv, CH), stream, (const T*)q,
                      q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache,
-                     block_table, table_stride, token_req, positions, nq, nkv, d, dv, P, window, scale, sink, score_bias);
+                     block_table, table_stride, token_req, positions, nq, nkv, d, dv, P, window, scale, sink, score_bias,
+                     softcap, bucket_of, far, rel);
 }
 
 // Whether the kernel takes this group and head size at all (0 and the reason in tk_last_error
@@ -179,7 +185,9 @@ TK_API int tk_paged_attention_generic(int dt, const void* q, int q_stride, void*
                                           const int* block_table, int table_stride,
                                           const int* token_req, const int* positions, int n_tokens,
                                           int nq, int nkv, int d, int dv, int P, int window, float scale,
-                                          const float* sink, const float* score_bias, hipStream_t stream) {
+                                          const float* sink, const float* score_bias, float softcap,
+                                          const int* bucket_of, int far, const float* rel, hipStream_t stream) {
+  TK_REQUIRE(!rel || (bucket_of && far >= 0), "paged_attention: a bias by distance needs its table of buckets");
   TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && P > 0 && nq % nkv == 0,
              "paged_attention: bad sizes tokens=%d nq=%d nkv=%d d=%d dv=%d P=%d", n_tokens, nq, nkv, d, dv,
              P);
@@ -197,7 +205,8 @@ TK_API int tk_paged_attention_generic(int dt, const void* q, int q_stride, void*
              "paged_attention: head size %d with group %d does not fit the local memory", d, group);
 #define AG_CASE(T, CHV)                                                                         \
   ag_launch<T, CHV>(q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride,    \
-                    token_req, positions, n_tokens, nq, nkv, d, dv, P, window, scale, sink, score_bias, stream)
+                    token_req, positions, n_tokens, nq, nkv, d, dv, P, window, scale, sink, score_bias, softcap, \
+                    bucket_of, far, rel, stream)
   if (dt == TK_F32) {
     if (ch == 64) AG_CASE(float, 64);
     else if (ch == 32) AG_CASE(float, 32);

@@ -71,6 +71,21 @@ __device__ __forceinline__ float gate_of(const AfterSum<T>& after, int tok, int 
   return after.gate ? 1.0f / (1.0f + expf(-to_f32<T>(after.gate[(size_t)tok * after.gate_stride + head]))) : 1.f;
 }
 
+// What may happen to a score between the scaling and the softmax, for mixers that ask for it: a soft cap
+// (score <- cap * tanh(score / cap), cap > 0) and then a learned bias by distance, rel[bucket][head] with
+// bucket = bucket_of[min(query position - key position, far)] (a table that the host made).
+struct ScoreShape {
+  float softcap;
+  const int* bucket_of;
+  int far;
+  const float* rel;
+};
+__device__ __forceinline__ float shaped_score(const ScoreShape& sh, float s, int dist, int head, int nq) {
+  if (sh.softcap > 0.f) s = sh.softcap * tanhf(s / sh.softcap);
+  if (sh.rel) s += sh.rel[(size_t)sh.bucket_of[min(max(dist, 0), sh.far)] * nq + head];
+  return s;
+}
+
 // SPLIT: the NW wavefronts of a workgroup share one tile and take its key steps in turn
 // (wavefront w the steps w, w + NW, ..); they add up through LDS, always in wavefront order.
 // For steps of few tiles (single decoded tokens), whose walks would else be one long chain each.
@@ -85,8 +100,8 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     const T* __restrict__ vcache, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
     const int* __restrict__ tile_row0, int nq, int nkv, int dk, int dv, int P, int window, float scale,
-    const float* __restrict__ sink, const float* __restrict__ score_bias, int gg, AfterSum<T> after, int chunk = 0,
-    float* __restrict__ part = nullptr) {
+    const float* __restrict__ sink, const float* __restrict__ score_bias, int gg, AfterSum<T> after, ScoreShape shape,
+    int chunk = 0, float* __restrict__ part = nullptr) {
   extern __shared__ float merge[];  // SPLIT: [waves][16] maxima, [waves][16] sums, [waves - 1][VT][4][64] weighted values
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
   const int group = nq / nkv;
@@ -142,6 +157,7 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
 #pragma unroll
   for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
   const bool sig = score_bias != nullptr;
+  const bool shaped = shape.softcap > 0.f || shape.rel != nullptr;
   const float pb = sig && live ? score_bias[head] : 0.f;
   // (sigmoid weights have no maximum to follow: it stays 0, so every merge below multiplies by exp(0))
   float m_run = sig ? 0.f : -INFINITY, l_run = 0.f;  // l_run: this lane's share of the column's sum
@@ -229,6 +245,7 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         sc[i] = s[i] * scale;
+        if (shaped) sc[i] = shaped_score(shape, sc[i], pos - (k0 + 4 * c + i), head, nq);
         tmax = fmaxf(tmax, sc[i]);
       }
     } else {
@@ -236,7 +253,7 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
       for (int i = 0; i < 4; ++i) {
         const int kp = k0 + 4 * c + i;
         const bool seen = live && kp <= pos && (window <= 0 || pos - kp < window);
-        sc[i] = seen ? s[i] * scale : -INFINITY;
+        sc[i] = seen ? (shaped ? shaped_score(shape, s[i] * scale, pos - kp, head, nq) : s[i] * scale) : -INFINITY;
         tmax = fmaxf(tmax, sc[i]);
       }
     }
@@ -480,7 +497,8 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
                       const void* kcache, const void* vcache, const int* block_table, int table_stride,
                       const int* q_start, const int* kv_len, const int* tile_req, const int* tile_row0, int nq,
                       int nkv, int dk, int dv, int P, int window, float scale, const float* sink, const float* score_bias,
-                      int gg, int chunk, float* part, const float* vfreq, int v_pair_half, const void* gate, int gate_stride) {
+                      int gg, int chunk, float* part, const float* vfreq, int v_pair_half, const void* gate, int gate_stride,
+                      ScoreShape shape) {
   // halves of a head meet inside a lane only where the head fills the kernel's blocks of 16 (the entry point has checked)
   const AfterSum<T> after = {vfreq, v_pair_half, (const T*)gate, gate_stride};
   const AfterSum<T> none = {nullptr, 0, nullptr, 0};
@@ -490,7 +508,7 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW, true>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
                        table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg,
-                       none, chunk, part);
+                       none, shape, chunk, part);
     hipLaunchKernelGGL((attention_tile_merge_kernel<T, VT>), dim3(grid.x, grid.y), dim3(VT * TK_WAVE), 0, stream, part, (int)grid.z,
                        (T*)out, out_stride, q_start, tile_req, tile_row0, nq, nkv, dv, sink, gg, score_bias ? 1 : 0, kv_len, after);
   } else if (split) {
@@ -499,11 +517,11 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
     const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
-                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, after);
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, after, shape);
   } else {
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, false, AT_WAVES>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
-                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, after);
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, after, shape);
   }
 }
 
@@ -514,7 +532,11 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
                                  const int* kv_len, const int* tile_req, const int* tile_row0, int n_tiles, int nq,
                                  int nkv, int dk, int dv, int P, int window, float scale, const float* sink,
                                  const float* score_bias, int gg, int split, int chunk, int chunks, float* part,
-                                 const float* vfreq, int v_pair_half, const void* gate, int gate_stride, hipStream_t stream) {
+                                 const float* vfreq, int v_pair_half, const void* gate, int gate_stride, float softcap,
+                                 const int* bucket_of, int far, const float* rel, hipStream_t stream) {
+  TK_REQUIRE(!rel || (bucket_of && far >= 0), "attention_tile_f32: a bias by distance needs its table of buckets");
+  TK_REQUIRE(!(score_bias && (rel || softcap > 0.f)), "attention_tile_f32: sigmoid weights take neither a soft cap nor a bias by distance");
+  const ScoreShape shape = {softcap, bucket_of, far, rel};
   TK_REQUIRE(tk_attention_tile_f32_fits(nq, nkv, dk, dv, P), "attention_tile_f32: shape nq=%d nkv=%d dk=%d dv=%d P=%d not taken",
              nq, nkv, dk, dv, P);
   const int group = nq / nkv;
@@ -534,7 +556,7 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
   TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
 #define AT_ARGS grid, sp, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \
                 tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, score_bias, gg, parts ? chunk : 0, part, vfreq, v_pair_half, \
-                gate, gate_stride
+                gate, gate_stride, shape
 #define AT_VT(T, KMV)                                      \
   do {                                                     \
     if (vt <= 2) at_launch<T, KMV, 2>(AT_ARGS);            \

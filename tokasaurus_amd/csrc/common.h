@@ -141,3 +141,26 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   for (int w = 1; w < nwaves; ++w) total = fmaxf(total, scratch[w]);
   return total;
 }
+
+// Sums over the 16 lanes of a row of the wavefront through the lanes' own data paths (no LDS): partners
+// exchange and add, so every lane ends with the same bits, in an order that depends on nothing.
+__device__ __forceinline__ float dpp_quad_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_quad_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_half_mirror(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_row_mirror(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+}
+// the sum over the 16 lanes of a row, in every lane
+__device__ __forceinline__ float row_sum16(float v) {
+  v += dpp_quad_xor1(v);
+  v += dpp_quad_xor2(v);
+  v += dpp_half_mirror(v);
+  v += dpp_row_mirror(v);
+  return v;
+}

@@ -141,27 +141,6 @@ __global__ void delta_tail_kernel(const T* __restrict__ proj, int ld, int taps, 
 // The sums through the lanes use the lanes' own data paths (no LDS): partners exchange and
 // add, so every lane ends with the same bits, in an order that depends on nothing.
 // --------------------------------------------------------------------------
-__device__ __forceinline__ float dpp_quad_xor1(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float dpp_quad_xor2(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float dpp_half_mirror(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float dpp_row_mirror(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
-}
-// the sum over the 16 lanes of a row, in every lane
-__device__ __forceinline__ float row_sum16(float v) {
-  v += dpp_quad_xor1(v);
-  v += dpp_quad_xor2(v);
-  v += dpp_half_mirror(v);
-  v += dpp_row_mirror(v);
-  return v;
-}
-
 // Rows of tokens t0 .. t0 + nt - 1 into a buffer [nt][q | k | decay (dkp each) | v (cols) | beta | padding], by
 // `nmove` threads of which this is `me`.  Several loads are in flight a thread before the first is stored.
 // VEC: the three long pieces move 16 bytes at a time (the caller found sizes and offsets to be multiples of 4).

@@ -303,6 +303,31 @@ static void launch_clamped_glu(const void* gate_up, void* out, int rows, int int
                        (const T*)gate_up, (T*)out, inter, limit, alpha);
 }
 
+// gelu(gate) * up with the tanh form of gelu, [rows, 2I] laid out [gate | up] -> [rows, I]; 32-bit arithmetic, one rounding
+__device__ __forceinline__ float gelu_tanh_f32(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+template <typename T>
+__global__ void gelu_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+  const T* g = gu + (size_t)blockIdx.y * 2 * inter;
+  const T* u = g + inter;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < inter) out[(size_t)blockIdx.y * inter + i] = from_f32<T>(gelu_tanh_f32(to_f32<T>(g[i])) * to_f32<T>(u[i]));
+}
+
+TK_API int tk_gelu_glu(int dt, const void* gate_up, void* out, int rows, int inter, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && inter > 0, "gelu_glu: bad sizes %d %d", rows, inter);
+  TK_REQUIRE(rows < 65536, "gelu_glu: %d rows are too many for one call", rows);
+  if (rows == 0) return 0;
+  const dim3 grid((inter + 255) / 256, rows);
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(gelu_glu_kernel<float>, grid, dim3(256), 0, stream, (const float*)gate_up, (float*)out, inter);
+  else
+    hipLaunchKernelGGL(gelu_glu_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)gate_up, (bf16_t*)out, inter);
+  TK_CHECK_LAUNCH("gelu_glu");
+  return 0;
+}
+
 TK_API int tk_clamped_glu(int dt, const void* gate_up, void* out, int rows, int inter, float limit, float alpha,
                           hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && inter > 0 && limit > 0.f, "clamped_glu: bad sizes %d %d or limit", rows, inter);

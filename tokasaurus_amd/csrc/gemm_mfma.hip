@@ -75,6 +75,7 @@ struct GemmArgs {
   // the gated epilogue's other form (glu_limit > 0): g = min(gate, limit), u = clamp(up, -limit, limit),
   // g * sigmoid(glu_alpha * g) * (u + 1), 32-bit until the one rounding at the store
   float glu_limit, glu_alpha;
+  int glu_gelu;  // the gated epilogue's third form: gelu(gate) * up with the tanh form of gelu
   float out_scale;  // the 32-bit epilogue multiplies its result by this (1: as it is)
   int M, N, K;  // N: outputs (for SwiGLU the intermediate size; W then has 2N rows, gate first)
   int TH;       // weight rows of a tile that are used (16, or 8 to make twice the workgroups of a narrow output)
@@ -99,6 +100,9 @@ __device__ __forceinline__ void store4(const GemmArgs& a, f32x4_t v, f32x4_t up,
         const float gc = fminf(round_to<bf16_t>(g), a.glu_limit);
         const float uc = fminf(fmaxf(round_to<bf16_t>(u), -a.glu_limit), a.glu_limit);
         o[j] = gc / (1.0f + expf(-a.glu_alpha * gc)) * (uc + 1.0f);
+      } else if (a.glu_gelu) {
+        const float gr = round_to<bf16_t>(g);
+        o[j] = 0.5f * gr * (1.0f + tanhf(0.7978845608028654f * (gr + 0.044715f * gr * gr * gr))) * round_to<bf16_t>(u);
       } else {
         o[j] = silu_mul_bf16(g, u);
       }
@@ -692,6 +696,8 @@ struct GemmExtra {
   float glu_limit, glu_alpha;
   // a factor on the 32-bit epilogue's result; 0 stands for none
   float out_scale;
+  // the gated epilogue as gelu(gate) * up (tanh form); 0: not
+  int glu_gelu;
 };
 
 // Number of partial sums a row gets from the residual epilogue with emit_w: one a tile.
@@ -770,7 +776,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
     a.kcache = (bf16_t*)extra->kcache; a.vcache = (bf16_t*)extra->vcache;
     a.nq = extra->nq; a.nkv = extra->nkv; a.d = extra->d; a.P = extra->P;
     a.bias = (const bf16_t*)extra->bias;
-    a.glu_limit = extra->glu_limit; a.glu_alpha = extra->glu_alpha;
+    a.glu_limit = extra->glu_limit; a.glu_alpha = extra->glu_alpha; a.glu_gelu = extra->glu_gelu;
     if (extra->out_scale != 0.f) a.out_scale = extra->out_scale;
     norm = a.sumsq_in != nullptr;
   }

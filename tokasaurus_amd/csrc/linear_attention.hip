@@ -1,0 +1,298 @@
+// Linear attention with a decay, as a recurrence over the tokens of each request, and what stands
+// around it in the mixers that use it: the short causal convolution that is added to a mixer's input,
+// the norm of the recurrence's result (head by head or over all heads) with an optional sigmoid gate,
+// and a sigmoid gate on the rows of another mixer.
+//
+// Per head, with a matrix S [dk][dv] kept per request in 32-bit:
+//     S_t = diag(a_t) S_(t-1) + k_t v_t^T        o_t = S_t^T q_t
+// in two forms, both read from the 32-bit sums `proj` of one stacked product:
+//   LA_CONSTANT  q = silu(.), k = silu(.), v = silu(.), a_t = decay[head] for every row and token
+//   LA_FORGET    q = silu(.), f = low + (1 - low) * sigmoid(. + bias) per head and row of S; a_t = f, k_t = 1 - f; v as it is
+// Everything from the sums on (activations, gates, the state, the read-out) is 32-bit arithmetic.
+//
+// The state row of a slot is [H][dv][dk]: a value column's dk numbers lie together.  The columns of S
+// do not meet: a column is owned by LA_LANES neighbouring lanes that cut dk between them (lane l holds rows
+// l + LA_LANES * n) and add up through the wavefront's own data paths, always in the same order, so a
+// token's result does not depend on how its request's tokens were cut into steps or on what shares the batch.
+#include "common.h"
+
+#define LA_LANES 16
+#define LA_COLS 16     // value columns a workgroup owns (LA_COLS * LA_LANES threads)
+#define LA_TOKENS 16   // tokens staged in LDS at a time
+enum { LA_CONSTANT = 0, LA_FORGET = 1 };
+
+__device__ __forceinline__ float la_silu(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float la_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// Workgroup (head, request, block of LA_COLS value columns).  A chunk of tokens is staged as
+// [tokens][q | k | a (dkp each)][v (LA_COLS)], activations applied on the way in.
+template <int NQ, int MODE>
+__global__ __launch_bounds__(LA_COLS * LA_LANES) void linear_attention_kernel(
+    const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
+    const float* __restrict__ f_bias, const float* __restrict__ f_low, float* __restrict__ state, size_t state_stride,
+    const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ o, int H, int dk, int dv) {
+  constexpr int dkp = NQ * LA_LANES;
+  constexpr int row_floats = 3 * dkp + LA_COLS;
+  __shared__ float stage[LA_TOKENS * row_floats];
+  const int h = blockIdx.x, r = blockIdx.y;
+  const int col0 = blockIdx.z * LA_COLS;
+  const int lane = threadIdx.x % LA_LANES, grp = threadIdx.x / LA_LANES;
+  const int col = col0 + grp;
+  const bool live = col < dv;
+  const int first = q_start[r], last = q_start[r + 1];
+  float* s_col = state + (size_t)slots[r] * state_stride + ((size_t)h * dv + (live ? col : 0)) * dk;
+  float s[NQ];
+#pragma unroll
+  for (int n = 0; n < NQ; ++n) {
+    const int i = lane + LA_LANES * n;
+    s[n] = (live && i < dk) ? s_col[i] : 0.f;
+  }
+  const float a_head = MODE == LA_CONSTANT ? decay[h] : 0.f;
+#pragma unroll 1
+  for (int t0 = first; t0 < last; t0 += LA_TOKENS) {
+    const int nt = min(LA_TOKENS, last - t0);
+    __syncthreads();  // the chunk before is consumed
+    for (int x = threadIdx.x; x < nt * row_floats; x += blockDim.x) {
+      const int tt = x / row_floats, rem = x % row_floats;
+      const float* row = proj + (size_t)(t0 + tt) * ld;
+      float val = 0.f;
+      if (rem < 3 * dkp) {
+        const int which = rem / dkp, i = rem % dkp;
+        if (i < dk) {
+          const int c = h * dk + i;
+          if (MODE == LA_CONSTANT) {
+            val = which == 0 ? la_silu(row[q_off + c]) : (which == 1 ? la_silu(row[k_off + c]) : a_head);
+          } else {
+            if (which == 0) {
+              val = la_silu(row[q_off + c]);
+            } else {
+              const float lo = f_low[c];
+              const float f = lo + (1.0f - lo) * la_sigmoid(row[k_off + c] + f_bias[c]);
+              val = which == 1 ? 1.0f - f : f;
+            }
+          }
+        }
+      } else {
+        const int c = col0 + rem - 3 * dkp;
+        if (c < dv) {
+          const float v = row[v_off + h * dv + c];
+          val = MODE == LA_CONSTANT ? la_silu(v) : v;
+        }
+      }
+      stage[x] = val;
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int tt = 0; tt < nt; ++tt) {
+      const float* row = stage + tt * row_floats;
+      const float v = row[3 * dkp + grp];
+      float acc = 0.f;
+#pragma unroll
+      for (int n = 0; n < NQ; ++n) {
+        const int i = lane + LA_LANES * n;
+        s[n] = fmaf(row[2 * dkp + i], s[n], row[dkp + i] * v);
+        acc = fmaf(row[i], s[n], acc);
+      }
+      acc = row_sum16(acc);
+      if (live && lane == 0) o[(size_t)(t0 + tt) * H * dv + (size_t)h * dv + col] = acc;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+      const int i = lane + LA_LANES * n;
+      if (i < dk) s_col[i] = s[n];
+    }
+  }
+}
+
+TK_API int tk_linear_attention(int mode, const float* proj, int ld, int q_off, int k_off, int v_off, const float* decay,
+                               const float* f_bias, const float* f_low, float* state, size_t state_stride,
+                               const int* q_start, const int* slots, float* o, int n_requests, int H, int dk, int dv,
+                               hipStream_t stream) {
+  TK_REQUIRE(n_requests >= 0 && H > 0 && dk > 0 && dv > 0 && dk <= 16 * LA_LANES,
+             "linear_attention: bad sizes requests=%d heads=%d dk=%d dv=%d (dk up to %d)", n_requests, H, dk, dv, 16 * LA_LANES);
+  TK_REQUIRE(mode == LA_CONSTANT ? decay != nullptr : (mode == LA_FORGET && f_bias && f_low),
+             "linear_attention: the constant form needs a decay a head, the forget-gate form a bias and a lower bound");
+  TK_REQUIRE(proj && state && q_start && slots && o && state_stride >= (size_t)H * dk * dv && n_requests < 65536,
+             "linear_attention: a pointer is missing, the state's rows are too short or the requests too many");
+  if (n_requests == 0) return 0;
+  const int nq = (dk + LA_LANES - 1) / LA_LANES;
+  const dim3 grid(H, n_requests, (dv + LA_COLS - 1) / LA_COLS), block(LA_COLS * LA_LANES);
+#define LA_CASE(NQ)                                                                                                              \
+  do {                                                                                                                           \
+    if (mode == LA_CONSTANT)                                                                                                     \
+      hipLaunchKernelGGL((linear_attention_kernel<NQ, LA_CONSTANT>), grid, block, 0, stream, proj, ld, q_off, k_off, v_off,      \
+                         decay, f_bias, f_low, state, state_stride, q_start, slots, o, H, dk, dv);                               \
+    else                                                                                                                         \
+      hipLaunchKernelGGL((linear_attention_kernel<NQ, LA_FORGET>), grid, block, 0, stream, proj, ld, q_off, k_off, v_off, decay, \
+                         f_bias, f_low, state, state_stride, q_start, slots, o, H, dk, dv);                                      \
+  } while (0)
+  if (nq <= 1) LA_CASE(1);
+  else if (nq <= 2) LA_CASE(2);
+  else if (nq <= 4) LA_CASE(4);
+  else if (nq <= 8) LA_CASE(8);
+  else LA_CASE(16);
+#undef LA_CASE
+  TK_CHECK_LAUNCH("linear_attention");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// Behind the recurrence: every group's `size` numbers of a token divided by their root mean square, times a
+// weight [size] that the groups share, times sigmoid(gate) where there is a gate, times `scale`; rounded once
+// to T.  A group is a head (a norm head by head) or the whole row (groups = 1).  A wavefront a (token, group).
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ld_gate,
+                                                              int groups, const float* __restrict__ w, float eps, float scale,
+                                                              T* __restrict__ out, int ld_out, long units, int size) {
+  const int lane = threadIdx.x & (TK_WAVE - 1);
+  const long unit = (long)blockIdx.x * (blockDim.x / TK_WAVE) + threadIdx.x / TK_WAVE;
+  if (unit >= units) return;
+  const long t = unit / groups;
+  const int g = (int)(unit % groups);
+  const float* x = o + (size_t)unit * size;
+  float ss = 0.f;
+  for (int i = lane; i < size; i += TK_WAVE) ss = fmaf(x[i], x[i], ss);
+  ss = wave_sum(ss);
+  const float rstd = 1.0f / sqrtf(ss / (float)size + eps);
+  for (int i = lane; i < size; i += TK_WAVE) {
+    float y = x[i] * rstd * w[i];
+    if (gate) y *= la_sigmoid(gate[(size_t)t * ld_gate + (size_t)g * size + i]);
+    out[(size_t)t * ld_out + (size_t)g * size + i] = from_f32<T>(y * scale);
+  }
+}
+
+TK_API int tk_group_norm_gate(int dt, const float* o, const float* gate, int ld_gate, const float* w, float eps, float scale,
+                              void* out, int ld_out, int n_tokens, int groups, int size, hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && groups > 0 && size > 0 && o && w && out, "group_norm_gate: bad sizes %d %d %d or a pointer is missing",
+             n_tokens, groups, size);
+  TK_REQUIRE(ld_out >= groups * size && (!gate || ld_gate >= groups * size), "group_norm_gate: a row stride is too short");
+  if (n_tokens == 0) return 0;
+  const long units = (long)n_tokens * groups;
+  const long blocks = (units + 3) / 4;
+  TK_REQUIRE(blocks < (1l << 31), "group_norm_gate: too many rows");
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(group_norm_gate_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, o, gate, ld_gate, groups, w, eps,
+                       scale, (float*)out, ld_out, units, size);
+  else
+    hipLaunchKernelGGL(group_norm_gate_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, o, gate, ld_gate, groups, w, eps,
+                       scale, (bf16_t*)out, ld_out, units, size);
+  TK_CHECK_LAUNCH("group_norm_gate");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// out[t, i] = x[t, i] * sigmoid(gate[t, i]) * scale, element by element (rows a stride apart), 32-bit arithmetic,
+// one rounding.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void sigmoid_gate_kernel(const T* __restrict__ x, int ld_x, const T* __restrict__ gate, int ld_gate, float scale,
+                                    T* __restrict__ out, int ld_out, int width) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t t = blockIdx.y;
+  if (i < width)
+    out[t * ld_out + i] = from_f32<T>(to_f32<T>(x[t * ld_x + i]) * la_sigmoid(to_f32<T>(gate[t * ld_gate + i])) * scale);
+}
+
+TK_API int tk_sigmoid_gate(int dt, const void* x, int ld_x, const void* gate, int ld_gate, float scale, void* out, int ld_out,
+                           int rows, int width, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && rows < 65536 && width > 0 && x && gate && out && ld_x >= width && ld_gate >= width && ld_out >= width,
+             "sigmoid_gate: bad sizes %d %d, a pointer is missing or a stride is too short", rows, width);
+  if (rows == 0) return 0;
+  const dim3 grid((width + 255) / 256, rows);
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, ld_x, (const float*)gate, ld_gate,
+                       scale, (float*)out, ld_out, width);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)x, ld_x, (const bf16_t*)gate, ld_gate,
+                       scale, (bf16_t*)out, ld_out, width);
+  TK_CHECK_LAUNCH("sigmoid_gate");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// A short causal convolution over time on every channel, added to its input:
+//     out_t = h_t + sum_j w[c][j] * h_(t - taps + 1 + j)      (zeros before a request's first token)
+// The last taps - 1 inputs of a request live in its slot's `tail` [taps - 1][width] (32-bit, oldest first,
+// zeros when the request takes the slot).  A thread a (token, channel).  FUSE_TAIL (every request of the step
+// brings one token): the thread also moves its channel's tail on, which it alone reads; else the tail kernel
+// below runs afterwards.
+// --------------------------------------------------------------------------
+#define SC_MAX_TAPS 16
+template <typename T, bool FUSE_TAIL>
+__global__ void short_conv_kernel(const T* __restrict__ h, int ld, const float* __restrict__ w, int taps, float* __restrict__ tails,
+                                  size_t tail_stride, const int* __restrict__ q_start, const int* __restrict__ token_req,
+                                  const int* __restrict__ slots, T* __restrict__ out, int width) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int r = token_req[t];
+  const int first = q_start[r];
+  const int local = t - first;
+  float* tail = tails + (size_t)slots[r] * tail_stride;
+  float acc = 0.f, cur = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = local - (taps - 1) + j;
+    const float x = src >= 0 ? to_f32<T>(h[(size_t)(first + src) * ld + c]) : tail[(size_t)(src + taps - 1) * width + c];
+    acc = fmaf(w[(size_t)c * taps + j], x, acc);
+    cur = x;
+    if (FUSE_TAIL && j >= 1) tail[(size_t)(j - 1) * width + c] = x;  // (local is 0: entry j - 1 was read a tap ago)
+  }
+  out[(size_t)t * width + c] = from_f32<T>(cur + acc);
+}
+
+// The tails after the step: the last taps - 1 inputs of every request, from this step's rows and, where the
+// step brought fewer, from the old tail.  A thread a (request, channel); it reads all it needs before it writes.
+template <typename T>
+__global__ void short_conv_tail_kernel(const T* __restrict__ h, int ld, int taps, float* __restrict__ tails, size_t tail_stride,
+                                       const int* __restrict__ q_start, const int* __restrict__ slots, int width) {
+  const int r = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int first = q_start[r], n = q_start[r + 1] - first;
+  float* tail = tails + (size_t)slots[r] * tail_stride;
+  float keep[SC_MAX_TAPS];
+#pragma unroll
+  for (int s = 0; s < SC_MAX_TAPS - 1; ++s) {
+    if (s < taps - 1) {
+      const int src = n - (taps - 1) + s;
+      keep[s] = src >= 0 ? to_f32<T>(h[(size_t)(first + src) * ld + c]) : tail[(size_t)(src + taps - 1) * width + c];
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < SC_MAX_TAPS - 1; ++s)
+    if (s < taps - 1) tail[(size_t)s * width + c] = keep[s];
+}
+
+TK_API int tk_short_conv(int dt, const void* h, int ld, const float* w, int taps, float* tails, size_t tail_stride,
+                         const int* q_start, const int* token_req, const int* slots, void* out, int n_tokens, int n_requests,
+                         int width, int single_tokens, hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && n_requests >= 0 && width > 0 && taps >= 1 && taps <= SC_MAX_TAPS && ld >= width,
+             "short_conv: bad sizes tokens=%d requests=%d width=%d taps=%d", n_tokens, n_requests, width, taps);
+  TK_REQUIRE(h && w && out && q_start && token_req && slots && (taps == 1 || (tails && tail_stride >= (size_t)(taps - 1) * width)),
+             "short_conv: a pointer is missing or the tails' rows are too short");
+  TK_REQUIRE(n_tokens < 65536 * 32 && n_requests < 65536, "short_conv: too many rows for one call");
+  if (n_tokens == 0) return 0;
+  TK_REQUIRE(n_tokens < 65536, "short_conv: %d tokens are too many for one call", n_tokens);
+  const dim3 grid((width + 255) / 256, n_tokens), tail_grid((width + 255) / 256, n_requests);
+#define SC_CASE(T)                                                                                                                   \
+  do {                                                                                                                               \
+    if (single_tokens)                                                                                                               \
+      hipLaunchKernelGGL((short_conv_kernel<T, true>), grid, dim3(256), 0, stream, (const T*)h, ld, w, taps, tails, tail_stride,     \
+                         q_start, token_req, slots, (T*)out, width);                                                                 \
+    else {                                                                                                                           \
+      hipLaunchKernelGGL((short_conv_kernel<T, false>), grid, dim3(256), 0, stream, (const T*)h, ld, w, taps, tails, tail_stride,    \
+                         q_start, token_req, slots, (T*)out, width);                                                                 \
+      if (taps > 1)                                                                                                                  \
+        hipLaunchKernelGGL(short_conv_tail_kernel<T>, tail_grid, dim3(256), 0, stream, (const T*)h, ld, taps, tails, tail_stride,    \
+                           q_start, slots, width);                                                                                   \
+    }                                                                                                                                \
+  } while (0)
+  if (dt == TK_F32) SC_CASE(float);
+  else SC_CASE(bf16_t);
+#undef SC_CASE
+  TK_CHECK_LAUNCH("short_conv");
+  return 0;
+}

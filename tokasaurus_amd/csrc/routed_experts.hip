@@ -70,13 +70,14 @@ __device__ __forceinline__ void wave_dot2(const T* __restrict__ w0, const T* __r
 // --------------------------------------------------------------------------
 // The router.  One workgroup a token.  n_all = routed + identity experts.  ids [tokens, top] names
 // the chosen experts in the order of their choice scores, weights [tokens, top] their softmax
-// scores (the correction moves the choice, not the weight).
+// scores (the correction moves the choice, not the weight); with `norm_scale` != 0 the chosen scores divided by
+// their sum (+ 1e-20) and multiplied by norm_scale.  Without `w_gate` a given `shared_gate` is filled with ones.
 // --------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(1024) void expert_route_kernel(
     const T* __restrict__ h, int h_stride, const T* __restrict__ w_router, const float* __restrict__ correction,
     const T* __restrict__ w_gate, int width, int n_all, int groups, int keep, int top, int* __restrict__ ids,
-    float* __restrict__ weights, float* __restrict__ shared_gate) {
+    float* __restrict__ weights, float* __restrict__ shared_gate, float norm_scale) {
   extern __shared__ float sm[];
   float* score = sm;                 // [n_all] logits, then softmax scores
   float* choice = sm + n_all;        // [n_all] score + correction, -inf outside the kept groups and once taken
@@ -84,6 +85,7 @@ __global__ __launch_bounds__(1024) void expert_route_kernel(
   const int t = blockIdx.x;
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE, nwaves = blockDim.x / TK_WAVE;
   const T* row = h + (size_t)t * h_stride;
+  if (!w_gate && shared_gate && threadIdx.x == 0) shared_gate[t] = 1.f;
   for (int e = wave; e < n_all + (w_gate ? 1 : 0); e += nwaves) {
     const float d = wave_dot<T>(e < n_all ? w_router + (size_t)e * width : w_gate, row, width);
     if (lane == 0) {
@@ -152,11 +154,16 @@ __global__ __launch_bounds__(1024) void expert_route_kernel(
     }
     __syncthreads();
   }
+  if (norm_scale != 0.f && threadIdx.x == 0) {
+    float sum = 0.f;
+    for (int r = 0; r < top; ++r) sum += weights[(size_t)t * top + r];
+    for (int r = 0; r < top; ++r) weights[(size_t)t * top + r] = weights[(size_t)t * top + r] / (sum + 1e-20f) * norm_scale;
+  }
 }
 
 TK_API int tk_expert_route(int dt, const void* h, int h_stride, const void* w_router, const float* correction,
                            const void* w_gate, int tokens, int width, int n_all, int groups, int keep, int top,
-                           int* ids, float* weights, float* shared_gate, hipStream_t stream) {
+                           int* ids, float* weights, float* shared_gate, float norm_scale, hipStream_t stream) {
   TK_REQUIRE(tokens >= 0 && width > 0 && n_all > 0 && groups > 0 && n_all % groups == 0 && keep > 0 && keep <= groups &&
                  top > 0 && top <= n_all,
              "expert_route: bad sizes tokens=%d width=%d experts=%d groups=%d keep=%d top=%d", tokens, width, n_all,
@@ -171,11 +178,11 @@ TK_API int tk_expert_route(int dt, const void* h, int h_stride, const void* w_ro
   if (dt == TK_F32)
     hipLaunchKernelGGL(expert_route_kernel<float>, dim3(tokens), dim3(threads), smem, stream, (const float*)h, h_stride,
                        (const float*)w_router, correction, (const float*)w_gate, width, n_all, groups, keep, top, ids,
-                       weights, shared_gate);
+                       weights, shared_gate, norm_scale);
   else
     hipLaunchKernelGGL(expert_route_kernel<bf16_t>, dim3(tokens), dim3(threads), smem, stream, (const bf16_t*)h, h_stride,
                        (const bf16_t*)w_router, correction, (const bf16_t*)w_gate, width, n_all, groups, keep, top, ids,
-                       weights, shared_gate);
+                       weights, shared_gate, norm_scale);
   TK_CHECK_LAUNCH("expert_route");
   return 0;
 }

@@ -8,33 +8,91 @@
 
 // --------------------------------------------------------------------------
 // out[t, :] = float(table[id_t, :]) * scale; id_t < 0 names slot -id_t-1 of `last_token`.
+// `pos_table` (null or [n_pos, hidden]): the learned row of the token's position is added, as it is.
 // --------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_scaled_kernel(const int* __restrict__ ids, const int* __restrict__ last_token,
                                     const T* __restrict__ table, float* __restrict__ out, int hidden,
-                                    int vocab, float scale) {
+                                    int vocab, float scale, const T* __restrict__ pos_table,
+                                    const int* __restrict__ positions, int n_pos) {
   const int t = blockIdx.x;
   int id = ids[t];
   if (id < 0) id = last_token[-id - 1];
   id = min(max(id, 0), vocab - 1);
   const T* src = table + (size_t)id * hidden;
   float* dst = out + (size_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32<T>(src[i]) * scale;
+  if (pos_table) {
+    const T* add = pos_table + (size_t)min(max(positions[t], 0), n_pos - 1) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = fmaf(to_f32<T>(src[i]), scale, to_f32<T>(add[i]));
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32<T>(src[i]) * scale;
+  }
 }
 
 TK_API int tk_embed_scaled(int dt, const int* ids, const int* last_token, const void* table,
                            float* out, int n_tokens, int hidden, int vocab, float scale,
-                           hipStream_t stream) {
+                           const void* pos_table, const int* positions, int n_pos, hipStream_t stream) {
   TK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_scaled: bad sizes %d %d %d", n_tokens,
              hidden, vocab);
+  TK_REQUIRE(!pos_table || (positions && n_pos > 0), "embed_scaled: a table of positions needs the tokens' positions");
   if (n_tokens == 0) return 0;
   if (dt == TK_F32)
     hipLaunchKernelGGL(embed_scaled_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, ids,
-                       last_token, (const float*)table, out, hidden, vocab, scale);
+                       last_token, (const float*)table, out, hidden, vocab, scale, (const float*)pos_table, positions, n_pos);
   else
     hipLaunchKernelGGL(embed_scaled_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, ids,
-                       last_token, (const bf16_t*)table, out, hidden, vocab, scale);
+                       last_token, (const bf16_t*)table, out, hidden, vocab, scale, (const bf16_t*)pos_table, positions, n_pos);
   TK_CHECK_LAUNCH("embed_scaled");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// A weighted sum over the streams a model has had so far, row by row:
+//     out[r, :] = sum_{j < count} w[j] * hist[j][row(r), :]  (+ w[count] * last[r, :])
+// `hist` holds `count` streams of equal shape `stride` floats apart; row(r) = rows[r] where `rows` is given
+// (the streams then have more rows than the result: only some are wanted), else r.  `last` (or null) is one
+// more stream that already has the result's rows.  For a norm that reads the result (`nw`, or null) the row
+//     out / sqrt(mean(out^2) + eps) * (offset + nw)
+// is written too, rounded once to T.  One row a workgroup; the sum runs over j in ascending order.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void depth_average_kernel(const float* __restrict__ hist, size_t stride, int count,
+                                                            const float* __restrict__ last, const int* __restrict__ rows,
+                                                            const float* __restrict__ w, float* __restrict__ out,
+                                                            const float* __restrict__ nw, float offset, float eps,
+                                                            T* __restrict__ normed, int hidden) {
+  __shared__ float red[16];
+  const size_t r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : r;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < count; ++j) acc = fmaf(w[j], hist[(size_t)j * stride + src * hidden + i], acc);
+    if (last) acc = fmaf(w[count], last[r * hidden + i], acc);
+    out[r * hidden + i] = acc;
+    ss = fmaf(acc, acc, ss);
+  }
+  if (!nw) return;
+  ss = block_sum(ss, red);
+  const float rstd = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)  // a thread reads back what it wrote
+    normed[r * hidden + i] = from_f32<T>(out[r * hidden + i] * rstd * (offset + nw[i]));
+}
+
+TK_API int tk_depth_average(int dt, const float* hist, size_t stride, int count, const float* last, const int* rows,
+                            const float* w, float* out, const float* nw, float offset, float eps, void* normed,
+                            int n_rows, int hidden, hipStream_t stream) {
+  TK_REQUIRE(n_rows >= 0 && hidden > 0 && count >= 0 && (count > 0 || last) && w && out && (count == 0 || hist),
+             "depth_average: bad sizes rows=%d hidden=%d streams=%d or a pointer is missing", n_rows, hidden, count);
+  TK_REQUIRE(!nw || normed, "depth_average: a norm's weight needs a place for its rows");
+  if (n_rows == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(depth_average_kernel<float>, dim3(n_rows), dim3(256), 0, stream, hist, stride, count, last, rows, w, out,
+                       nw, offset, eps, (float*)normed, hidden);
+  else
+    hipLaunchKernelGGL(depth_average_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, stream, hist, stride, count, last, rows, w, out,
+                       nw, offset, eps, (bf16_t*)normed, hidden);
+  TK_CHECK_LAUNCH("depth_average");
   return 0;
 }
 

@@ -28,7 +28,7 @@ CSRC = Path(__file__).resolve().parent.parent / "csrc"
 IN_TREE_DIR = Path(__file__).resolve().parent / "_build"
 GROUPS = {
     "core": ["errors.hip", "elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sample.hip", "step_io.hip",
-             "stream_f32.hip", "attention_prepare.hip", "attention_tile_f32.hip", "delta_rule.hip", "routed_experts.hip", "gated_recurrence.hip"],
+             "stream_f32.hip", "attention_prepare.hip", "attention_tile_f32.hip", "delta_rule.hip", "routed_experts.hip", "gated_recurrence.hip", "linear_attention.hip"],
     "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip", "grouped_gemm.hip"],
     "library": ["errors.hip", "gemm_library.hip"],
 }

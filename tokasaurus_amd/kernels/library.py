@@ -35,10 +35,16 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_head_rmsnorm": [c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P],
         "tk_paged_attention_generic": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P]
         + [c_int] * 7
-        + [c_float, _P, _P, _P],
+        + [c_float, _P, _P, c_float, _P, c_int, _P, _P],
         "tk_paged_attention_generic_fits": [c_int, c_int, c_int, c_int],
         "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
-        "tk_embed_scaled": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
+        "tk_embed_scaled": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, _P, c_int, _P],
+        "tk_depth_average": [c_int, _P, c_size_t, c_int, _P, _P, _P, _P, _P, c_float, c_float, _P, c_int, c_int, _P],
+        "tk_linear_attention": [c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, c_size_t, _P, _P, _P] + [c_int] * 4 + [_P],
+        "tk_group_norm_gate": [c_int, _P, _P, c_int, _P, c_float, c_float, _P, c_int, c_int, c_int, c_int, _P],
+        "tk_sigmoid_gate": [c_int, _P, c_int, _P, c_int, c_float, _P, c_int, c_int, c_int, _P],
+        "tk_short_conv": [c_int, _P, c_int, _P, c_int, _P, c_size_t, _P, _P, _P, _P] + [c_int] * 4 + [_P],
+        "tk_gelu_glu": [c_int, _P, _P, c_int, c_int, _P],
         "tk_residual_norm": [c_int, _P, _P, _P, c_float, _P, _P, _P, c_float, c_float, _P, _P, c_int, c_int, _P],
         "tk_softcap": [_P, c_size_t, c_float, _P],
         "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 13 + [_P, c_int, c_float, _P],
@@ -51,13 +57,13 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_gather_keys": [c_int, _P, _P, c_int, _P, _P, _P] + [c_int] * 5 + [_P],
         "tk_post_norm_residual": [c_int, _P, _P, _P, c_float, _P, _P, c_float, _P, c_int, c_int, _P],
         "tk_concat_cast": [c_int, _P, _P, _P, c_int, c_int, _P],
-        "tk_expert_route": [c_int, _P, c_int, _P, _P, _P] + [c_int] * 6 + [_P, _P, _P, _P],
+        "tk_expert_route": [c_int, _P, c_int, _P, _P, _P] + [c_int] * 6 + [_P, _P, _P, c_float, _P],
         "tk_expert_gate_up": [c_int, _P, c_int, _P, _P, _P] + [c_int] * 5 + [_P],
         "tk_expert_combine": [c_int, _P, c_int, _P, _P, _P, _P, _P, _P, _P] + [c_int] * 5 + [_P],
         "tk_head_linear": [c_int, _P, c_int, _P, _P, c_int, c_int] + [c_int] * 4 + [_P],
         "tk_squared_relu": [c_int, _P, c_size_t, _P],
         "tk_attention_tile_f32": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P] + [c_int] * 7
-        + [c_float, _P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, _P, c_int, _P],
+        + [c_float, _P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, _P, c_int, c_float, _P, c_int, _P, _P],
         "tk_attention_tile_turns_halves": [c_int],
         "tk_attention_tile_part_words": [c_int],
         "tk_attention_tile_f32_fits": [c_int] * 5,

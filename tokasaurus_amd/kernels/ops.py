@@ -356,14 +356,19 @@ def paged_attention_generic(
     value_dim: int | None = None,
     sink: torch.Tensor | None = None,
     score_bias: torch.Tensor | None = None,
+    softcap: float = 0.0,
+    distance_bias: "DistanceBias | None" = None,
 ) -> torch.Tensor:
     """Attention of every token over its request's pages (see rope_append for
     the page layout).  ``q`` is 2-d, its first nq*d columns are the query heads.
     ``value_dim``: the size of a value head (a key head's by default); the result is
     [tokens, nq * value_dim].  ``sink`` (32-bit, one number a query head): exp(sink) joins the
     softmax's denominator once, with no key and no value.  ``score_bias`` (32-bit, one number a
-    query head): no softmax; a visible key's weight is sigmoid(score + score_bias[head]), not normalised."""
+    query head): no softmax; a visible key's weight is sigmoid(score + score_bias[head]), not normalised.
+    ``softcap`` (> 0): a scaled score becomes softcap * tanh(score / softcap).  ``distance_bias``: a learned
+    number by (bucket of the distance, head) is added to the score after that."""
     _gpu(q, kcache, vcache, block_table, token_req, positions, sink, score_bias)
+    db = _checked_distance_bias(distance_bias, nq)
     vd = head_dim if value_dim is None else int(value_dim)
     _f32_vector(score_bias, nq, "attention: the scores' biases")
     _need(sink is None or (sink.shape == (nq,) and sink.dtype == torch.float32 and sink.is_contiguous()),
@@ -401,9 +406,45 @@ def paged_attention_generic(
         float(scale if scale is not None else 1.0 / math.sqrt(head_dim)),
         sink.data_ptr() if sink is not None else None,
         score_bias.data_ptr() if score_bias is not None else None,
+        float(softcap), *db,
         _stream(),
     )
     return out
+
+
+@dataclass
+class DistanceBias:
+    """A learned bias on attention scores by distance: ``rel`` [buckets, heads] (32-bit) and ``bucket_of``
+    [far + 1] (int32), the bucket of every distance up to ``far``, which stands for all beyond it."""
+
+    rel: torch.Tensor
+    bucket_of: torch.Tensor
+
+
+def distance_buckets(buckets: int, far: int) -> list[int]:
+    """The bucket of every distance 0 .. far: distances below half the buckets have one each, the others
+    share the rest on a logarithmic scale that reaches the last bucket at ``far``."""
+    half = buckets // 2
+    _need(buckets >= 2 and far > half, "distance_buckets: at least two buckets, and distances beyond half of them")
+    out = []
+    for n in range(int(far) + 1):
+        if n < half:
+            out.append(n)
+        else:
+            out.append(min(buckets - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (buckets - half)))))
+    return out
+
+
+def _checked_distance_bias(db: "DistanceBias | None", nq: int) -> tuple:
+    """The kernels' three arguments for a bias by distance (null pointers without one)."""
+    if db is None:
+        return None, 0, None
+    _gpu(db.rel, db.bucket_of)
+    _i32(db.bucket_of, "the distances' buckets")
+    _need(db.rel.dim() == 2 and db.rel.shape[1] == nq and db.rel.dtype == torch.float32 and db.rel.is_contiguous(),
+          f"attention: the bias by distance must be contiguous float32 [buckets, {nq}]")
+    _need(db.bucket_of.numel() >= 1, "attention: the table of buckets is empty")
+    return db.bucket_of.data_ptr(), db.bucket_of.numel() - 1, db.rel.data_ptr()
 
 
 def paged_attention_generic_fits(nq: int, nkv: int, head_dim: int, value_dim: int | None = None) -> bool:
@@ -839,7 +880,7 @@ class _GemmExtra(ctypes.Structure):
         ("kcache", ctypes.c_void_p), ("vcache", ctypes.c_void_p),
         ("nq", ctypes.c_int), ("nkv", ctypes.c_int), ("d", ctypes.c_int), ("P", ctypes.c_int),
         ("bias", ctypes.c_void_p), ("glu_limit", ctypes.c_float), ("glu_alpha", ctypes.c_float),
-        ("out_scale", ctypes.c_float),
+        ("out_scale", ctypes.c_float), ("glu_gelu", ctypes.c_int),
     ]
 
 
@@ -920,7 +961,10 @@ def gemm_skinny_bf16(
         n //= 2
         n_out = n
         epi = EPI_SWIGLU
-        if glu is not None:
+        if glu == "gelu_tanh":  # gelu(gate) * up
+            extra.glu_gelu = 1
+            use_extra = True
+        elif glu is not None:
             _need(glu[0] > 0, "gemm_skinny: the clamp's limit must be positive")
             extra.glu_limit, extra.glu_alpha = float(glu[0]), float(glu[1])
             use_extra = True
@@ -1112,10 +1156,17 @@ def _f32_vector(t: torch.Tensor | None, n: int, name: str) -> None:
         raise KernelError(f"{name} must be contiguous float32 [{n}]")
 
 
-def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, last_token: torch.Tensor | None = None) -> torch.Tensor:
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, last_token: torch.Tensor | None = None,
+                 pos_table: torch.Tensor | None = None, positions: torch.Tensor | None = None) -> torch.Tensor:
     """out[t] = float32(table[ids[t]]) * scale: the first rows of a 32-bit residual stream;
-    ids[t] < 0 reads the token from last_token[-ids[t]-1]."""
-    _gpu(ids, table, last_token)
+    ids[t] < 0 reads the token from last_token[-ids[t]-1].  ``pos_table`` [positions, H] of the table's type:
+    the row of the token's position (``positions``) is added, as it is."""
+    _gpu(ids, table, last_token, pos_table, positions)
+    if pos_table is not None:
+        _need(pos_table.dim() == 2 and pos_table.is_contiguous() and pos_table.shape[1] == table.shape[1] and pos_table.dtype == table.dtype,
+              "embed_scaled: the table of positions must be contiguous [positions, H] of the embedding's type")
+        _i32(positions, "positions")
+        _need(positions.numel() == ids.numel(), "embed_scaled: one position a token")
     _i32(ids, "ids")
     _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [V, H]")
     if last_token is not None:
@@ -1124,7 +1175,163 @@ def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, last_toke
     vocab, hidden = table.shape
     out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
     call("tk_embed_scaled", dtype_code(table.dtype), ids.data_ptr(), last_token.data_ptr() if last_token is not None else None,
-         table.data_ptr(), out.data_ptr(), n, hidden, vocab, float(scale), _stream())
+         table.data_ptr(), out.data_ptr(), n, hidden, vocab, float(scale),
+         pos_table.data_ptr() if pos_table is not None else None, positions.data_ptr() if pos_table is not None else None,
+         pos_table.shape[0] if pos_table is not None else 0, _stream())
+    return out
+
+
+def depth_average(hist: torch.Tensor, count: int, weights: torch.Tensor, last: torch.Tensor | None = None,
+                  rows: torch.Tensor | None = None, out: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None,
+                  unit_offset: bool = False, eps: float = 0.0, out_dtype: torch.dtype = torch.float32
+                  ) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """A weighted sum over the streams a model has had so far: ``hist`` [streams, tokens, H] (32-bit) of which the
+    first ``count`` count, ``weights`` (32-bit, one number a stream, ``last``'s behind the others); ``rows`` (int32):
+    only these rows of the streams are wanted, in this order; ``last`` [len(rows) or tokens, H]: one more stream that
+    already has the result's rows.  ``out``: where the result goes (a contiguous 32-bit buffer of its shape).
+    ``norm_weight`` (32-bit [H]): also returns the result's rows through an RMS norm with this weight (plus one
+    with ``unit_offset``), rounded once to ``out_dtype``."""
+    _gpu(hist, weights, last, rows, out, norm_weight)
+    _need(hist.dim() == 3 and hist.dtype == torch.float32 and hist.is_contiguous() and 0 <= count <= hist.shape[0],
+          "depth_average: the streams must be contiguous float32 [streams, tokens, H]")
+    hidden = hist.shape[2]
+    n = rows.numel() if rows is not None else (last.shape[0] if last is not None else hist.shape[1])
+    if rows is not None:
+        _i32(rows, "rows")
+    _need(last is None or (last.shape == (n, hidden) and last.dtype == torch.float32 and last.is_contiguous()),
+          "depth_average: the last stream must be contiguous float32 with the result's rows")
+    _need(rows is not None or n == hist.shape[1], "depth_average: without chosen rows every stream has the result's rows")
+    _f32_vector(weights, count + (1 if last is not None else 0), "depth_average: the weights")
+    _f32_vector(norm_weight, hidden, "depth_average: a norm weight")
+    if out is None:
+        out = torch.empty((n, hidden), dtype=torch.float32, device=hist.device)
+    _need(out.shape == (n, hidden) and out.dtype == torch.float32 and out.is_contiguous(), "depth_average: the result's buffer")
+    normed = torch.empty((n, hidden), dtype=out_dtype, device=hist.device) if norm_weight is not None else None
+    if n:
+        call("tk_depth_average", dtype_code(out_dtype), hist.data_ptr(), hist.stride(0), int(count),
+             last.data_ptr() if last is not None else None, rows.data_ptr() if rows is not None else None, weights.data_ptr(),
+             out.data_ptr(), norm_weight.data_ptr() if norm_weight is not None else None, 1.0 if unit_offset else 0.0, float(eps),
+             normed.data_ptr() if normed is not None else None, n, hidden, _stream())
+    return out, normed
+
+
+# --------------------------------------------------------------------------
+# linear attention with a decay, and what stands around it
+# --------------------------------------------------------------------------
+
+def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: torch.Tensor, q_start: torch.Tensor,
+                     slots: torch.Tensor, heads: int, key_dim: int, value_dim: int, decay: torch.Tensor | None = None,
+                     forget_bias: torch.Tensor | None = None, forget_low: torch.Tensor | None = None) -> torch.Tensor:
+    """The recurrence ``S_t = diag(a_t) S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t`` per head over every request's
+    tokens of this step, from the 32-bit sums ``proj`` of one stacked product (columns from ``q_off``, ``k_off``
+    and ``v_off`` on, head by head).  With ``decay`` (32-bit, one number a head): q, k and v pass silu and a_t is
+    the head's decay.  With ``forget_bias`` and ``forget_low`` (32-bit [heads * key_dim]): q passes silu, the
+    columns at ``k_off`` are a forget gate's, f = low + (1 - low) * sigmoid(. + bias), a_t = f and k_t = 1 - f, v as
+    it is.  ``state`` [slots + 1, heads * value_dim * key_dim] (32-bit) is read and written in the requests'
+    ``slots``.  Returns o [tokens, heads * value_dim] in 32-bit."""
+    _gpu(proj, state, q_start, slots, decay, forget_bias, forget_low)
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1, "linear_attention: 32-bit rows with unit inner stride")
+    H, dk, dv = int(heads), int(key_dim), int(value_dim)
+    n, width = proj.shape
+    for off, size in ((q_off, H * dk), (k_off, H * dk), (v_off, H * dv)):
+        _need(0 <= off and off + size <= width, "linear_attention: a part lies outside the rows")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] >= H * dk * dv,
+          "linear_attention: the state must be contiguous float32 [slots, heads * dv * dk]")
+    _i32(q_start, "q_start")
+    _i32(slots, "slots")
+    _need(q_start.numel() == slots.numel() + 1, "linear_attention: one slot a request")
+    constant = decay is not None
+    _need(constant != (forget_bias is not None and forget_low is not None), "linear_attention: a decay a head, or a forget gate's bias and bound")
+    _f32_vector(decay, H, "linear_attention: the decays")
+    _f32_vector(forget_bias, H * dk, "linear_attention: the forget gate's bias")
+    _f32_vector(forget_low, H * dk, "linear_attention: the forget gate's lower bound")
+    o = torch.empty((n, H * dv), dtype=torch.float32, device=proj.device)
+    if n:
+        call("tk_linear_attention", 0 if constant else 1, proj.data_ptr(), proj.stride(0), int(q_off), int(k_off), int(v_off),
+             decay.data_ptr() if constant else None, forget_bias.data_ptr() if not constant else None,
+             forget_low.data_ptr() if not constant else None, state.data_ptr(), state.stride(0), q_start.data_ptr(),
+             slots.data_ptr(), o.data_ptr(), slots.numel(), H, dk, dv, _stream())
+    return o
+
+
+def group_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, out_dtype: torch.dtype,
+                    gate: torch.Tensor | None = None, scale: float = 1.0, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Every group's numbers of a token (``groups`` equal groups a row of the 32-bit ``o``) divided by their root
+    mean square, times ``weight`` (32-bit, one group's size, shared by the groups), times sigmoid(``gate``) where
+    one is given (32-bit, ``o``'s shape, rows a stride apart), times ``scale``; rounded once to ``out_dtype``.
+    ``out``: a 2-d view of that type to write to (rows a stride apart)."""
+    _gpu(o, weight, gate, out)
+    _need(o.dim() == 2 and o.dtype == torch.float32 and o.is_contiguous() and o.shape[1] % groups == 0,
+          "group_norm_gate: contiguous float32 rows of equal groups")
+    n, width = o.shape
+    size = width // int(groups)
+    _f32_vector(weight, size, "group_norm_gate: the weight")
+    _need(gate is None or (gate.shape == o.shape and gate.dtype == torch.float32 and gate.stride(1) == 1),
+          "group_norm_gate: a 32-bit gate of the rows' shape")
+    if out is None:
+        out = torch.empty((n, width), dtype=out_dtype, device=o.device)
+    _need(out.shape == (n, width) and out.dtype == out_dtype and out.stride(1) == 1, "group_norm_gate: the result's view")
+    if n:
+        call("tk_group_norm_gate", dtype_code(out_dtype), o.data_ptr(), gate.data_ptr() if gate is not None else None,
+             gate.stride(0) if gate is not None else 0, weight.data_ptr(), float(eps), float(scale), out.data_ptr(), out.stride(0),
+             n, int(groups), size, _stream())
+    return out
+
+
+def sigmoid_gate(x: torch.Tensor, gate: torch.Tensor, scale: float = 1.0, out: torch.Tensor | None = None) -> torch.Tensor:
+    """x * sigmoid(gate) * scale element by element (2-d views of one type and shape, rows a stride apart), 32-bit
+    arithmetic, one rounding; into ``out`` (such a view) or a new tensor."""
+    _gpu(x, gate, out)
+    _need(x.dim() == 2 and gate.shape == x.shape and gate.dtype == x.dtype and x.stride(1) == 1 and gate.stride(1) == 1,
+          "sigmoid_gate: rows and gates of one shape and type with unit inner stride")
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _need(out.shape == x.shape and out.dtype == x.dtype and out.stride(1) == 1, "sigmoid_gate: the result's view")
+    n, width = x.shape
+    for first in range(0, n, 65535):
+        m = min(65535, n - first)
+        xs, gs, os_ = x[first : first + m], gate[first : first + m], out[first : first + m]
+        call("tk_sigmoid_gate", dtype_code(x.dtype), xs.data_ptr(), x.stride(0), gs.data_ptr(), gate.stride(0), float(scale),
+             os_.data_ptr(), out.stride(0), m, width, _stream())
+    return out
+
+
+def short_conv(h: torch.Tensor, weight: torch.Tensor, tails: torch.Tensor | None, q_start: torch.Tensor, token_req: torch.Tensor,
+               slots: torch.Tensor, single_tokens: bool) -> torch.Tensor:
+    """h + conv(h) with a causal convolution over time on every channel, ``conv(h)_t = sum_j weight[:, j] *
+    h_(t - taps + 1 + j)``, zeros before a request's start.  ``weight`` [width, taps] in 32-bit; ``tails``
+    [slots + 1, (taps - 1) * width] (32-bit) holds every request's last taps - 1 inputs and is moved on.
+    ``single_tokens``: every request of the step brings one token (the tails then move in the same kernel)."""
+    _gpu(h, weight, tails, q_start, token_req, slots)
+    _need(h.dim() == 2 and h.stride(1) == 1, "short_conv: rows with unit inner stride")
+    n, width = h.shape
+    _need(weight.dim() == 2 and weight.shape[0] == width and weight.dtype == torch.float32 and weight.is_contiguous(),
+          "short_conv: taps must be contiguous float32 [width, taps]")
+    taps = weight.shape[1]
+    if taps > 1:
+        _need(tails is not None and tails.dim() == 2 and tails.dtype == torch.float32 and tails.is_contiguous()
+              and tails.shape[1] >= (taps - 1) * width, "short_conv: the tails must be contiguous float32 [slots, (taps - 1) * width]")
+    for t, name in ((q_start, "q_start"), (token_req, "token_req"), (slots, "slots")):
+        _i32(t, name)
+    _need(token_req.numel() == n and q_start.numel() == slots.numel() + 1, "short_conv: one request a token, one slot a request")
+    out = torch.empty((n, width), dtype=h.dtype, device=h.device)
+    if n:
+        _need(n < 65536, "short_conv: a step of fewer than 65 536 tokens")
+        call("tk_short_conv", dtype_code(h.dtype), h.data_ptr(), h.stride(0), weight.data_ptr(), taps,
+             tails.data_ptr() if tails is not None else None, tails.stride(0) if tails is not None else 0, q_start.data_ptr(),
+             token_req.data_ptr(), slots.data_ptr(), out.data_ptr(), n, slots.numel(), width, 1 if single_tokens else 0, _stream())
+    return out
+
+
+def gelu_glu(gate_up: torch.Tensor) -> torch.Tensor:
+    """[rows, 2I] laid out [gate | up] -> gelu(gate) * up with the tanh form of gelu, [rows, I]; 32-bit arithmetic, one rounding."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gelu_glu input must be contiguous [rows, 2I]")
+    rows, two_i = gate_up.shape
+    out = torch.empty((rows, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    for first in range(0, rows, 65535):
+        m = min(65535, rows - first)
+        call("tk_gelu_glu", dtype_code(gate_up.dtype), gate_up[first:].data_ptr(), out[first:].data_ptr(), m, two_i // 2, _stream())
     return out
 
 
@@ -1407,7 +1614,8 @@ def attention_tile_f32(
     value_dim: int, page_size: int, heads_a_tile: int, window: int = 0, scale: float = 1.0,
     sink: torch.Tensor | None = None, split: bool | None = None, key_chunk: int = 0, longest: int = 0, first_row: int = 0,
     score_bias: torch.Tensor | None = None, value_freq: torch.Tensor | None = None,
-    value_pair_halves: bool = False, gate: torch.Tensor | None = None,
+    value_pair_halves: bool = False, gate: torch.Tensor | None = None, softcap: float = 0.0,
+    distance_bias: "DistanceBias | None" = None,
 ) -> torch.Tensor:
     """Attention in 32-bit arithmetic on the matrix cores: every token of the step over its
     request's pages; ``tile_req`` / ``tile_row0`` name each tile's request and its first token's
@@ -1423,6 +1631,7 @@ def attention_tile_f32(
     ``value_pair_halves``, ``gate``: what ``unrotate_gate_`` does, in the kernel's own epilogue (halves only where
     ``attention_tile_turns_halves``)."""
     _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink, score_bias, value_freq, gate)
+    db = _checked_distance_bias(distance_bias, nq)
     _f32_vector(value_freq, value_dim // 2, "attention: the values' frequencies")
     _need(value_freq is None or not value_pair_halves or attention_tile_turns_halves(value_dim),
           "attention: the halves of this value size are turned back by unrotate_gate_")
@@ -1468,7 +1677,7 @@ def attention_tile_f32(
          1 if split else 0, int(key_chunk) if chunks else 0, chunks, part.data_ptr() if part is not None else None,
          value_freq.data_ptr() if value_freq is not None else None, 1 if value_pair_halves else 0,
          (gate.data_ptr() - int(first_row) * gate.stride(0) * gate.element_size()) if gate is not None else None,
-         gate.stride(0) if gate is not None else 0, _stream())
+         gate.stride(0) if gate is not None else 0, float(softcap), *db, _stream())
     return out
 
 
@@ -1668,12 +1877,15 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, out_f32: bool = False) -> torc
 
 
 def expert_route(h: torch.Tensor, w_router: torch.Tensor, correction: torch.Tensor, groups: int, keep: int, top: int,
-                 w_gate: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+                 w_gate: torch.Tensor | None = None, normalize_scale: float | None = None,
+                 unit_gate: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
     """The router of a mixture of experts, 32-bit arithmetic: logits ``w_router h`` over all
     experts, their softmax s, the choice by ``s + correction`` among the experts of the ``keep``
     groups of neighbours (of ``groups`` equal ones) whose best choice score is largest, ties to the
     left.  Returns ids [tokens, top] int32 in the order of the choice scores, weights [tokens, top]
-    (the chosen experts' s), and, with ``w_gate`` [width], sigmoid(w_gate . h) [tokens]."""
+    (the chosen experts' s), and, with ``w_gate`` [width], sigmoid(w_gate . h) [tokens].  ``normalize_scale``: the
+    weights are divided by their sum (+ 1e-20) and multiplied by this number.  ``unit_gate`` (without ``w_gate``): the
+    third result is a gate of ones, for a shared expert that is added as it is."""
     _gpu(h, w_router, correction, w_gate)
     n_all, width = w_router.shape
     _need(h.dim() == 2 and h.stride(1) == 1 and h.shape[1] == width and w_router.dtype == h.dtype and w_router.is_contiguous(),
@@ -1684,12 +1896,13 @@ def expert_route(h: torch.Tensor, w_router: torch.Tensor, correction: torch.Tens
     n = h.shape[0]
     ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((n, top), dtype=torch.float32, device=h.device)
-    gate = torch.empty((n,), dtype=torch.float32, device=h.device) if w_gate is not None else None
+    gate = torch.empty((n,), dtype=torch.float32, device=h.device) if (w_gate is not None or unit_gate) else None
     if n == 0:
         return ids, weights, gate
     call("tk_expert_route", dtype_code(h.dtype), h.data_ptr(), h.stride(0), w_router.data_ptr(), correction.data_ptr(),
          w_gate.data_ptr() if w_gate is not None else None, n, width, n_all, int(groups), int(keep), int(top),
-         ids.data_ptr(), weights.data_ptr(), gate.data_ptr() if gate is not None else None, _stream())
+         ids.data_ptr(), weights.data_ptr(), gate.data_ptr() if gate is not None else None,
+         float(normalize_scale) if normalize_scale else 0.0, _stream())
     return ids, weights, gate
 
 

@@ -88,20 +88,54 @@ class CausalLM:
         order = self.spec.run_order
         last = len(order) - 1
         # a connector reads the embedding's output again; blocks may update the stream in place
-        x0 = x.clone() if self.connectors else None
+        x0 = x.clone() if any(not getattr(c, "takes_history", False) for c in self.connectors) else None
+        # connectors that read every stream so far: the embedding's output and each block's result are kept side by
+        # side, [streams, tokens, H]; a block updates its input in place, so its input is a copy in the next place
+        hist = None
+        if any(getattr(c, "takes_history", False) for c in self.connectors) and order:
+            if x.dtype != torch.float32:
+                raise TypeError("connectors over the model's streams so far run on a 32-bit stream")
+            hist = torch.empty((len(order) + 1, *x.shape), dtype=torch.float32, device=x.device)
+            hist[0].copy_(x)
+            hist[1].copy_(x)
+            x = hist[1]
         for i, entry in enumerate(order):
             rows = want_rows if i == last else None
             block = self.blocks[entry.layer]
             if entry.before is not None:
                 x, prepared = self.connectors[entry.before].forward(x, x0), None
+                if hist is not None:
+                    hist[i + 1].copy_(x)
+                    x = hist[i + 1]
+            reader = None  # the norm that reads the stream this entry leaves
+            if i == last:
+                reader = self.head.entry_norm()
+            elif order[i + 1].before is None:  # (else the stream changes before the next block reads it)
+                reader = self.blocks[order[i + 1].layer].entry_norm()
             if block.fuses_norm:
-                next_norm = self.blocks[order[i + 1].layer].entry_norm() if i < last else self.head.entry_norm()
-                if i < last and order[i + 1].before is not None:
-                    next_norm = None  # the stream changes before the next block reads it
-                out = block.forward(x, ctx, caches[i], states[i], rows, prepared=prepared, next_norm=next_norm)
+                # (a connector behind this block changes the stream before anything reads it)
+                out = block.forward(x, ctx, caches[i], states[i], rows, prepared=prepared,
+                                    next_norm=None if entry.after is not None else reader)
             else:
                 out = block.forward(x, ctx, caches[i], states[i], rows)
             x, prepared = stream_and_prepared(out)
+            if hist is not None:
+                whole = rows is None
+                if whole and x.data_ptr() != hist[i + 1].data_ptr():
+                    hist[i + 1].copy_(x)  # (a block that did not update its input in place)
+                after = self.connectors[entry.after] if entry.after is not None else None
+                if after is not None and getattr(after, "takes_history", False):
+                    out = after.forward_history(hist, i + 2 if whole else i + 1, None if whole else x, rows,
+                                                hist[i + 2] if (whole and i < last) else None, next_norm=reader)
+                    x, prepared = stream_and_prepared(out)
+                elif i < last:
+                    hist[i + 2].copy_(x)
+                    x = hist[i + 2]
+            elif entry.after is not None:
+                raise RuntimeError("a connector behind a run entry reads the model's streams so far (takes_history)")
+            tap = ctx.extras.get("model_tap")
+            if tap is not None:  # a list that collects the stream every run entry leaves (tests, debugging)
+                tap.append(x.clone())
         if last < 0 and want_rows is not None:
             x = ops.gather_rows(x, want_rows)
         if logits_out is None:

@@ -18,6 +18,8 @@ from tokasaurus_amd.config.taborax_config import TaboraxConfig
 from tokasaurus_amd.models.taborax import taborax_spec
 from tokasaurus_amd.config.sakevik_config import SakevikConfig
 from tokasaurus_amd.models.sakevik import sakevik_spec
+from tokasaurus_amd.config.sazilorn_config import SazilornConfig
+from tokasaurus_amd.models.sazilorn import sazilorn_spec
 from tokasaurus_amd.models.spec import ModelSpec
 
 
@@ -44,6 +46,7 @@ register_architecture(Architecture("llama", LlamaConfig.from_dict, llama_spec, c
 register_architecture(Architecture("kupuzen", KupuzenConfig.from_dict, kupuzen_spec, class_names=("Kupuzen",)))
 register_architecture(Architecture("taborax", TaboraxConfig.from_dict, taborax_spec, class_names=("Taborax",)))
 register_architecture(Architecture("sakevik", SakevikConfig.from_dict, sakevik_spec, class_names=("Sakevik",)))
+register_architecture(Architecture("sazilorn", SazilornConfig.from_dict, sazilorn_spec, class_names=("Sazilorn",)))
 
 
 def architecture_of(config_dict: dict[str, Any]) -> Architecture:

@@ -3,8 +3,9 @@ layers run.
 
 ``run_order`` is a list of entries; an entry names a layer (the same layer may
 be named twice: its weights are then used twice, each use with a cache of its
-own) and may name an earlier entry whose cache it reads instead of keeping one, and a
-connector that runs on the stream right before it.
+own) and may name an earlier entry whose cache it reads instead of keeping one, a
+connector that runs on the stream right before it, and one that runs right behind it on
+all the streams the model has had so far.
 """
 
 from __future__ import annotations
@@ -19,6 +20,7 @@ class RunEntry:
     layer: int
     cache_of: int | None = None  # index into run_order of the entry whose cache is read
     before: int | None = None  # index into ModelSpec.connectors of what runs on the stream right before this entry
+    after: int | None = None  # index into ModelSpec.connectors of what runs on the model's streams right behind this entry
 
 
 @dataclass(frozen=True)
@@ -38,8 +40,9 @@ class ModelSpec:
 
     def validate(self) -> None:
         for i, e in enumerate(self.run_order):
-            if e.before is not None and not 0 <= e.before < len(self.connectors):
-                raise ValueError(f"run entry {i} names connector {e.before}, the model has {len(self.connectors)}")
+            for c in (e.before, e.after):
+                if c is not None and not 0 <= c < len(self.connectors):
+                    raise ValueError(f"run entry {i} names connector {c}, the model has {len(self.connectors)}")
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"run entry {i} names layer {e.layer}, the model has {len(self.layers)}")
             if e.cache_of is not None:

@@ -1,7 +1,7 @@
 """Parts a model is put together from.  Importing the package registers the
 built-in parts under their names."""
 
-from tokasaurus_amd.parts import (attention, block, delta_rule, embedding, feedforward, grouped_attention, latent_attention, min_gru,  # noqa: F401
+from tokasaurus_amd.parts import (attention, block, delta_rule, embedding, feedforward, grouped_attention, latent_attention, linear_attention, min_gru, mixer_pair,  # noqa: F401
                                    norm, position, routed_experts)
 from tokasaurus_amd.parts.base import (  # noqa: F401
     BLOCKS,

@@ -28,6 +28,8 @@ NORM_OFFSET = "norm_offset"  # a norm's scale stored around zero (the norm multi
 VECTOR = "vector"  # a learned vector of another role (a sink, a rate, a step's bias): N(0, 0.5) when random
 CONV = "conv"  # the taps of short convolutions, [channels, taps]: N(0, 0.5) when random
 SMALL_VECTOR = "small_vector"  # a learned vector that nudges (a router's correction): N(0, 0.01) when random
+UNIT_INTERVAL = "unit_interval"  # a learned bound or rate between 0 and 1: uniform on (0.05, 0.95) when random
+AVERAGE_WEIGHT = "average_weight"  # the weights of an average over n things, [n]: 1 / n + N(0, 0.1 / n) when random
 INT_TABLE = "int_table"  # integer table: kept as int32
 
 

@@ -29,7 +29,9 @@ from tokasaurus_amd.parts.base import (
     StepContext,
     TensorSpec,
 )
+from tokasaurus_amd.parts.base import AVERAGE_WEIGHT
 from tokasaurus_amd.parts.linear import Linear, Placer
+from tokasaurus_amd.parts.short_conv import ShortConvResidual
 
 
 def build_with_shared(registry, spec: PartSpec, shared: dict):
@@ -124,7 +126,10 @@ class NormPair(Part):
 class ParallelResidualBlock(Block):
     """Mixer and feed-forward side by side on a 32-bit residual stream:
         x <- x + mult * (mixer(norm1(x)) + ff(norm2(x)))
-    both norms of the same x; ``feed_forward`` (and its norm) may be absent.  The stream is
+    both norms of the same x; ``feed_forward`` (and its norm) may be absent.  With ``shared_norm`` there is one
+    norm and both sublayers read its rows (``ff_norm`` is then absent).  ``input_conv`` (``{"taps": n, "name":
+    checkpoint name}``): what the mixer reads is first replaced by ``h + conv(h)``, a short causal convolution over
+    time on every channel whose last inputs are part of a request's state (the feed-forward reads h as it is).  The stream is
     32-bit whatever the storage type; the branches hand over their last products' 32-bit sums,
     and one kernel adds them to the stream and writes the rows of the norms that read the new
     stream (the next block's pair, or the head's norm).  The norms are ``stream_rmsnorm``s; the
@@ -133,9 +138,13 @@ class ParallelResidualBlock(Block):
     fuses_norm = True
 
     def __init__(self, mixer_norm: PartSpec, mixer: PartSpec, ff_norm: PartSpec | None = None,
-                 feed_forward: PartSpec | None = None, residual_mult: float = 1.0, shared: dict | None = None):
+                 feed_forward: PartSpec | None = None, residual_mult: float = 1.0, shared: dict | None = None,
+                 shared_norm: bool = False, input_conv: dict | None = None):
         shared = shared if shared is not None else {}
-        if (ff_norm is None) != (feed_forward is None):
+        self.shared_norm = bool(shared_norm)
+        if self.shared_norm and ff_norm is not None:
+            raise ValueError("sublayers that share one norm have no second one")
+        if not self.shared_norm and (ff_norm is None) != (feed_forward is None):
             raise ValueError("a feed-forward and its norm come together")
         self.mixer_norm = build_with_shared(NORMS, mixer_norm, shared)
         self.mixer = build_with_shared(MIXERS, mixer, shared)
@@ -143,9 +152,16 @@ class ParallelResidualBlock(Block):
         self.feed_forward = build_with_shared(FEED_FORWARDS, feed_forward, shared) if feed_forward is not None else None
         self.residual_mult = float(residual_mult)
         self.entry = NormPair(self.mixer_norm, self.ff_norm)
+        self.input_conv = None
+        if input_conv:
+            self.input_conv = ShortConvResidual(self.mixer_norm.size, int(input_conv["taps"]), input_conv["name"])
 
     def children(self) -> list[Part]:
-        return [c for c in (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward) if c is not None]
+        return [c for c in (self.mixer_norm, self.input_conv, self.mixer, self.ff_norm, self.feed_forward) if c is not None]
+
+    def state_needs(self):
+        conv = self.input_conv.state_need() if self.input_conv is not None else None
+        return ([conv] if conv is not None else []) + super().state_needs()
 
     def tensor_specs(self) -> list[TensorSpec]:
         return [s for c in self.children() for s in c.tensor_specs()]
@@ -164,7 +180,17 @@ class ParallelResidualBlock(Block):
             h1, h2 = prepared.normed
         else:
             h1, h2 = self.entry.forward_pair(x)
-        a = self.mixer.mix(h1, ctx, cache, state, rows, out_f32=True)
+        if self.shared_norm:
+            h2 = h1
+        hm = h1
+        if self.input_conv is not None:
+            tails = None
+            if self.input_conv.state_need() is not None:
+                # the convolution's last inputs come first among the block's states
+                tails, rest = (state[0], state[1:]) if isinstance(state, list) else (state, [])
+                state = None if not rest else (rest[0] if len(rest) == 1 else rest)
+            hm = self.input_conv.forward(h1, ctx, tails)
+        a = self.mixer.mix(hm, ctx, cache, state, rows, out_f32=True)
         if rows is not None:
             x = ops.gather_rows(x, rows)
             h2 = ops.gather_rows(h2, rows) if h2 is not None else None
@@ -349,3 +375,43 @@ class EmbeddingMix(Connector):
 
     def forward(self, x: torch.Tensor, x0: torch.Tensor) -> torch.Tensor:
         return self.proj(ops.concat_cast(x, x0, self.proj.weight.dtype), out_f32=True)
+
+
+@CONNECTORS.register("depth_average")
+class DepthAverage(Connector):
+    """x <- sum_j w[j] X_j over the embedding's output X_0 and the results X_1 .. X_n of every block that has run
+    so far (each block's result before any such average): what goes on to the next block, or to the head.  One
+    weight vector of n + 1 numbers, kept in 32-bit; the sum is 32-bit in ascending j.  A connector of this kind
+    runs behind a run entry (``models.spec.RunEntry.after``) and is handed the model's streams so far instead of
+    the stream and the embedding's output; where the next reader begins with an RMS norm of the stream, the same
+    pass writes that norm's rows."""
+
+    takes_history = True
+
+    def __init__(self, streams: int, name: str):
+        self.streams, self.name = int(streams), name
+        self.weight: torch.Tensor | None = None
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [TensorSpec(self.name, (self.streams,), AVERAGE_WEIGHT)]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.weight = placer.place(("vector_f32", self.name), lambda: tensors[self.name].to(torch.float32).contiguous().to(placer.device))
+
+    def forward_history(self, hist: torch.Tensor, count: int, last: torch.Tensor | None, rows: torch.Tensor | None,
+                        out: torch.Tensor | None, next_norm=None):
+        """``hist`` [streams, tokens, H]: X_0 .. X_(count - 1); ``last``: X_count where it has only the wanted
+        ``rows``.  Returns the new stream (in ``out`` when given), or (stream, ``Prepared``) for ``next_norm``."""
+        if count + (1 if last is not None else 0) != self.streams:
+            raise RuntimeError(f"a depth average over {self.streams} streams was handed {count + (1 if last is not None else 0)}")
+        reader = next_norm.first if isinstance(next_norm, NormPair) and next_norm.second is None else next_norm
+        if getattr(reader, "same_rule", None) is None:
+            reader = None
+        x, normed = ops.depth_average(hist, count, self.weight, last=last, rows=rows, out=out,
+                                      norm_weight=reader.weight if reader is not None else None,
+                                      unit_offset=reader.unit_offset if reader is not None else False,
+                                      eps=reader.eps if reader is not None else 0.0,
+                                      out_dtype=reader.out_dtype if reader is not None else torch.float32)
+        if reader is None:
+            return x
+        return x, Prepared(None, next_norm, (normed, None) if isinstance(next_norm, NormPair) else normed)

@@ -18,9 +18,16 @@ from tokasaurus_amd.parts.linear import Linear, Placer
 
 @EMBEDDINGS.register("token_embedding")
 class TokenEmbedding(Embedding):
-    def __init__(self, vocab_size: int, hidden_size: int, name: str, scale: float | None = None, stream_f32: bool = False):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, scale: float | None = None, stream_f32: bool = False,
+                 position_name: str | None = None, max_positions: int = 0):
         """``scale``: every row is multiplied by it.  ``stream_f32``: the rows leave in 32-bit
-        whatever the table's storage type (a model that keeps its residual stream in 32-bit)."""
+        whatever the table's storage type (a model that keeps its residual stream in 32-bit).
+        ``position_name``: a learned table [max_positions, hidden]; the row of a token's position
+        (counted from 0 in its request) is added to the token's row, unscaled."""
+        self.position_name, self.max_positions = position_name, int(max_positions)
+        if position_name and (not stream_f32 or self.max_positions <= 0):
+            raise ValueError("learned positions go with a 32-bit stream and a table of at least one position")
+        self.positions: torch.Tensor | None = None
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.name = name
@@ -31,17 +38,24 @@ class TokenEmbedding(Embedding):
         self.table: torch.Tensor | None = None
 
     def tensor_specs(self) -> list[TensorSpec]:
-        return [TensorSpec(self.name, (self.vocab_size, self.hidden_size), MATRIX)]
+        specs = [TensorSpec(self.name, (self.vocab_size, self.hidden_size), MATRIX)]
+        if self.position_name:
+            specs.append(TensorSpec(self.position_name, (self.max_positions, self.hidden_size), MATRIX))
+        return specs
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
         host = tensors[self.name]
         self.table = placer.place(
             ("row_major", self.name), lambda: host.to(dtype=placer.dtype).contiguous().to(placer.device)
         )
+        if self.position_name:
+            self.positions = placer.place(("row_major", self.position_name), lambda: tensors[self.position_name].to(
+                dtype=placer.dtype).contiguous().to(placer.device))
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         if self.stream_f32:
-            return ops.embed_scaled(ctx.token_ids, self.table, 1.0 if self.scale is None else self.scale, ctx.last_token)
+            return ops.embed_scaled(ctx.token_ids, self.table, 1.0 if self.scale is None else self.scale, ctx.last_token,
+                                    pos_table=self.positions, positions=ctx.positions if self.positions is not None else None)
         return ops.embed_gather(ctx.token_ids, self.table, ctx.last_token)
 
 

@@ -15,9 +15,13 @@ from tokasaurus_amd.parts.linear import Linear, Placer
 class SwiGLU(FeedForward):
     fuses_norm = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, names: dict[str, str]):
+    def __init__(self, hidden_size: int, intermediate_size: int, names: dict[str, str], activation: str = "silu"):
+        """``activation``: what the gate passes, "silu" or "gelu_tanh" (the tanh form of gelu)."""
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
+        if activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"a gated feed-forward's activation is silu or gelu_tanh, not {activation!r}")
+        self.glu = None if activation == "silu" else activation
         self.gate_up = Linear(hidden_size, [names["gate"], names["up"]], [intermediate_size] * 2)
         self.down = Linear(intermediate_size, [names["down"]], [hidden_size])
 
@@ -29,12 +33,12 @@ class SwiGLU(FeedForward):
         self.down.load(tensors, placer)
 
     def forward(self, h: torch.Tensor | Normed, residual: torch.Tensor, emit_norm=None):
-        return self.down.with_residual(self.gate_up(h, swiglu=True), residual, emit_norm)
+        return self.down.with_residual(self.gate_up(h, swiglu=True, glu=self.glu), residual, emit_norm)
 
     def transform(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
         """The feed-forward's own output, nothing added: for blocks that combine their branches
         themselves.  ``out_f32``: the down projection's 32-bit sums leave unrounded."""
-        return self.down(self.gate_up(h, swiglu=True), out_f32=out_f32)
+        return self.down(self.gate_up(h, swiglu=True, glu=self.glu), out_f32=out_f32)
 
 
 @FEED_FORWARDS.register("squared_relu")

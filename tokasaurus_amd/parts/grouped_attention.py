@@ -9,7 +9,8 @@ instead of neighbours, and values that are the keys themselves as projected, bef
 (the mixer then has no value tensor); biases on the projections; norms of queries and keys head by
 head with one weight for all heads; weights that are sigmoids of the biased scores instead of a
 softmax; values turned by their own position and the heads' results turned back by the query's; a
-sigmoid gate per head that reads the mixer's input.
+sigmoid gate per head that reads the mixer's input; a soft cap on the scaled scores; a learned bias on the
+scores by (bucket of the distance, head); a sigmoid gate per element of the heads' results.
 
 Scores, softmax weights, norms, angles and the rotation are 32-bit arithmetic in either storage
 type.  One kernel norms, rotates and appends (``ops.qk_prepare``); the attention itself runs on
@@ -84,6 +85,9 @@ class GroupedAttention(Mixer):
         score_bias_name: str | None = None,
         value_rotation: dict | None = None,
         gate_name: str | None = None,
+        softcap: float | None = None,
+        distance_bias: dict | None = None,
+        element_gate_name: str | None = None,
     ):
         """``names``: checkpoint names of the q, k, v, o matrices (k and v only with ``own_kv``).
         ``projection_norm``: ``{"q": name, "k": name, "eps": eps}``, weights of the whole
@@ -100,7 +104,20 @@ class GroupedAttention(Mixer):
         weight of a visible key is sigmoid(score + bias), not normalised over the keys (no softmax, no sink).
         ``value_rotation``: ``{"base": b, "pair_halves": bool}``; the value at position j is cached turned,
         pair m by j * b^(-2m/value_dim), and a head's result at position i is turned back by i.
-        ``gate_name``: a matrix [heads, hidden]; head h's result is multiplied by sigmoid(gate h)_h."""
+        ``gate_name``: a matrix [heads, hidden]; head h's result is multiplied by sigmoid(gate h)_h.
+        ``softcap``: a scaled score s becomes softcap * tanh(s / softcap).  ``distance_bias``: ``{"name": n, "buckets":
+        B, "far": D}``, a table [B, heads] of which row bucket(i - j) is added to the score of query i and key j (after
+        the scale and the soft cap): distances below B / 2 have a bucket each, the others share the rest on a
+        logarithmic scale that reaches the last bucket at D.  ``element_gate_name``: a matrix [heads * value_dim,
+        hidden]; the heads' results are multiplied element by element by sigmoid(gate h)."""
+        self.softcap = float(softcap) if softcap else 0.0
+        self.distance_bias = dict(distance_bias) if distance_bias else None
+        self.element_gate_name = element_gate_name
+        if score_bias_name and (self.softcap or self.distance_bias):
+            raise ValueError("sigmoid weights take neither a soft cap nor a bias by distance")
+        if element_gate_name and gate_name:
+            raise ValueError("a gate per head or a gate per element, not both")
+        self.rel: "ops.DistanceBias | None" = None
         self.key_chunk = int(key_chunk)
         bias_names = dict(bias_names or {})
         self.head_norm = dict(head_norm) if head_norm else None
@@ -138,6 +155,9 @@ class GroupedAttention(Mixer):
         biases = [bias_names.get("q")] + ([bias_names.get("k")] + ([] if self.values_are_keys else [bias_names.get("v")]) if own_kv else [])
         if gate_name:  # the gate reads the same input: one more part of the stacked product
             stacked, sizes, biases = stacked + [gate_name], sizes + [num_heads], biases + [None]
+        if element_gate_name:
+            stacked, sizes, biases = stacked + [element_gate_name], sizes + [num_heads * value_dim], biases + [None]
+        self.element_gate_col = sum(sizes) - num_heads * value_dim if element_gate_name else None
         self.gate_col = sum(sizes) - num_heads if gate_name else None
         self.qkv = Linear(hidden_size, stacked, sizes, bias_names=biases)
         self.out = Linear(num_heads * value_dim, [names["o"]], [hidden_size], bias_names=[bias_names.get("o")])
@@ -168,7 +188,13 @@ class GroupedAttention(Mixer):
             specs.append(TensorSpec(self.sink_name, (self.num_heads,), VECTOR))
         if self.score_bias_name:
             specs.append(TensorSpec(self.score_bias_name, (self.num_heads,), VECTOR))
+        if self.distance_bias:
+            specs.append(TensorSpec(self.distance_bias["name"], (int(self.distance_bias["buckets"]), self.num_heads), VECTOR))
         return specs
+
+    @property
+    def inner_size(self) -> int:
+        return self.num_heads * self.value_dim
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed(self.num_kv_heads, self.key_dim, self.cache_window,
@@ -195,6 +221,11 @@ class GroupedAttention(Mixer):
                 self.k_norm_weight = f32(self.head_norm["k"])
         if self.score_bias_name:
             self.score_bias = f32(self.score_bias_name)
+        if self.distance_bias:
+            buckets, far = int(self.distance_bias["buckets"]), int(self.distance_bias["far"])
+            table = placer.place(("distance_buckets", buckets, far), lambda: torch.tensor(
+                ops.distance_buckets(buckets, far), dtype=torch.int32).to(placer.device))
+            self.rel = ops.DistanceBias(f32(self.distance_bias["name"]), table)
         if self.value_rotation:
             dv, base = self.value_dim, float(self.value_rotation["base"])
             self.value_freq = placer.place(("value_freq", dv, base), lambda: torch.tensor(
@@ -207,7 +238,8 @@ class GroupedAttention(Mixer):
         if self.position is not None:
             self.position.prepare(placer.device)
 
-    def _attend(self, h: torch.Tensor, ctx: StepContext, cache: CacheView, rows: torch.Tensor | None) -> torch.Tensor:
+    def _attend(self, h: torch.Tensor, ctx: StepContext, cache: CacheView, rows: torch.Tensor | None,
+                out: torch.Tensor | None = None, out_scale: float = 1.0) -> torch.Tensor:
         assert cache is not None, "grouped attention needs a cache"
         if cache.writable != self.own_kv:
             raise RuntimeError("a mixer with key and value tensors of its own writes its cache; one without reads another's")
@@ -236,16 +268,25 @@ class GroupedAttention(Mixer):
                                           window=self.window, scale=self.scale, sink=self.sink, key_chunk=self.key_chunk,
                                           longest=ctx.extras.get("kv_bound", ctx.max_kv_len), score_bias=self.score_bias,
                                           value_freq=self.value_freq if fused else None, value_pair_halves=v_halves,
-                                          gate=gate if fused else None)
+                                          gate=gate if fused else None, softcap=self.softcap, distance_bias=self.rel)
             after = after and not fused
         else:  # sizes that the matrix-core kernel does not take
             attn = ops.paged_attention_generic(qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
                                                nq, nkv, dk, cache.page_size, window=self.window, scale=self.scale,
-                                               value_dim=dv, sink=self.sink, score_bias=self.score_bias)
+                                               value_dim=dv, sink=self.sink, score_bias=self.score_bias, softcap=self.softcap,
+                                               distance_bias=self.rel)
         if after:
             # the heads' results turned back by their own positions, then each head's gate
             ops.unrotate_gate_(attn, ctx.positions, self.value_freq, v_halves, gate, nq, dv)
+        if self.element_gate_col is not None:
+            attn = ops.sigmoid_gate(attn, qkv[:, self.element_gate_col : self.element_gate_col + nq * dv], scale=out_scale, out=out)
+        elif out is not None or out_scale != 1.0:
+            raise NotImplementedError("grouped attention gives its rows with a factor, or into a view, through its gate per element only")
         return attn if rows is None else ops.gather_rows(attn, rows)
+
+    def inner_rows(self, h, ctx, cache, state, out=None, scale: float = 1.0):
+        """The heads' results in front of the output projection times ``scale``, into ``out`` (a view) when given."""
+        return self._attend(h, ctx, cache, None, out=out, out_scale=scale)
 
     def mix(self, h, ctx, cache, state, rows, out_f32: bool = False):
         return self.out(self._attend(h, ctx, cache, rows), out_f32=out_f32)

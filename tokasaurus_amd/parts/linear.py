@@ -99,7 +99,7 @@ class Linear:
         rows: int | None = None,
         swiglu: bool = False,
         out: torch.Tensor | None = None,
-        glu: tuple[float, float] | None = None,
+        glu: "tuple[float, float] | str | None" = None,
         out_scale: float | None = None,
     ) -> torch.Tensor:
         """x [M, in] -> [M, out].  ``residual``: returns residual + product (the
@@ -109,12 +109,13 @@ class Linear:
         weight (a mixer that only needs its queries).  ``x`` may be a ``Normed``:
         the norm is folded into the product when it was prepared, else applied first.
         ``out`` (with ``out_f32``): a buffer [M, out] for the result, in place of new memory.
-        ``glu`` (with ``swiglu``): (limit, alpha) of the gated activation with clamps, in place of silu(gate) * up.
+        ``glu`` (with ``swiglu``): (limit, alpha) of the gated activation with clamps, or "gelu_tanh" for gelu(gate) * up
+        with the tanh form of gelu, in place of silu(gate) * up.
         ``out_scale`` (with ``out_f32``): the 32-bit result times this factor (in the few-row product's epilogue, else by a
         pass of its own)."""
         assert out_scale is None or (out_f32 and residual is None), "a factor on the result goes with 32-bit output"
         scaled = (lambda p: ops.scale_(p, out_scale)) if out_scale is not None and float(out_scale) != 1.0 else (lambda p: p)
-        gated = (lambda p: ops.clamped_glu(p, glu[0], glu[1])) if glu is not None else ops.swiglu
+        gated = ops.gelu_glu if glu == "gelu_tanh" else ((lambda p: ops.clamped_glu(p, glu[0], glu[1])) if glu is not None else ops.swiglu)
         assert out is None or (out_f32 and residual is None and not swiglu), "a result buffer goes with 32-bit output only"
         w, bias = self.weight, self.bias
         if rows is not None and rows != self.total_out:

@@ -5,10 +5,11 @@ experts together, ``s = softmax(logits)``; the choice is made by ``s + correctio
 vector that moves the choice and not the weight); the experts form ``groups`` equal groups of
 neighbours, a group's mark is its largest choice score, and only experts of the ``keep`` groups
 with the largest marks can be chosen; the ``top`` largest choice scores win and the chosen experts'
-``s`` are their weights, as they are.  A routed expert is ``W_down (silu(W_gate h) * (W_up h))``;
+``s`` are their weights, as they are or (``normalize_scale``) divided by their sum (+ 1e-20) and multiplied by a
+constant.  A routed expert is ``W_down (silu(W_gate h) * (W_up h))``;
 the last ``identity`` router outputs have no tensors, their output is ``h`` itself.  A shared
 expert of the same form may run for every token; its output is multiplied by
-``sigmoid(w_sg . h)``, one number a token, and added.
+``sigmoid(w_sg . h)``, one number a token, where the checkpoint has such a gate, and added.
 
 One kernel routes (and computes the shared expert's gate); the experts' products run pair by
 pair (token, chosen expert), each a function of its own token only, and are summed per token
@@ -27,12 +28,15 @@ from tokasaurus_amd.parts.linear import Linear, Placer
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(FeedForward):
     def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, names: dict[str, str],
-                 identity: int = 0, groups: int = 1, keep: int = 1, shared_size: int | None = None):
+                 identity: int = 0, groups: int = 1, keep: int = 1, shared_size: int | None = None,
+                 normalize_scale: float | None = None):
         """``names``: ``router`` ([experts + identity, hidden]), ``correction`` ([experts + identity]),
         ``expert``: a pattern with ``{e}`` for the expert's number that gives the prefix of its
         ``.gate``, ``.up`` ([expert_size, hidden]) and ``.down`` ([hidden, expert_size]); with a
-        shared expert also ``shared`` (the prefix of its three matrices) and ``shared_gate``
-        ([1, hidden])."""
+        shared expert also ``shared`` (the prefix of its three matrices) and, where it has a gate,
+        ``shared_gate`` ([1, hidden]).  ``normalize_scale``: the chosen experts' weights are divided by their sum
+        and multiplied by this number."""
+        self.normalize_scale = float(normalize_scale) if normalize_scale else None
         self.hidden_size, self.expert_size = hidden_size, int(expert_size)
         self.num_experts, self.top, self.identity = int(num_experts), int(top), int(identity)
         self.groups, self.keep = int(groups), int(keep)
@@ -60,7 +64,8 @@ class RoutedExperts(FeedForward):
                       TensorSpec(self._expert(e, "down"), (W, F), MATRIX)]
         if self.shared_size:
             specs += self.shared_gate_up.tensor_specs() + self.shared_down.tensor_specs()
-            specs.append(TensorSpec(self.names["shared_gate"], (1, W), MATRIX))
+            if self.names.get("shared_gate"):
+                specs.append(TensorSpec(self.names["shared_gate"], (1, W), MATRIX))
         return specs
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
@@ -79,10 +84,13 @@ class RoutedExperts(FeedForward):
         if self.shared_size:
             self.shared_gate_up.load(tensors, placer)
             self.shared_down.load(tensors, placer)
-            self.shared_gate = place(("row_major", n["shared_gate"]), lambda: tensors[n["shared_gate"]].to(placer.dtype).reshape(-1))
+            if n.get("shared_gate"):
+                self.shared_gate = place(("row_major", n["shared_gate"]), lambda: tensors[n["shared_gate"]].to(placer.dtype).reshape(-1))
 
     def transform(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
-        ids, weights, gate = ops.expert_route(h, self.router, self.correction, self.groups, self.keep, self.top, self.shared_gate)
+        ids, weights, gate = ops.expert_route(h, self.router, self.correction, self.groups, self.keep, self.top, self.shared_gate,
+                                              normalize_scale=self.normalize_scale,
+                                              unit_gate=bool(self.shared_size) and self.shared_gate is None)
         shared = self.shared_down(self.shared_gate_up(h, swiglu=True), out_f32=True) if self.shared_size else None
         y = ops.expert_mix(h, self.w_gate_up, self.w_down, ids, weights, shared, gate)
         return y if out_f32 else y.to(h.dtype)

@@ -20,7 +20,8 @@ import torch
 from safetensors.torch import save_file
 
 from tokasaurus_amd.models.registry import architecture_of
-from tokasaurus_amd.parts.base import BIAS, CONV, INT_TABLE, MATRIX, NORM_OFFSET, NORM_WEIGHT, SMALL_VECTOR, VECTOR, TensorSpec
+from tokasaurus_amd.parts.base import (AVERAGE_WEIGHT, BIAS, CONV, INT_TABLE, MATRIX, NORM_OFFSET, NORM_WEIGHT, SMALL_VECTOR, UNIT_INTERVAL,
+                                       VECTOR, TensorSpec)
 
 MATRIX_STD = 0.02
 NORM_STD = 0.01
@@ -48,6 +49,11 @@ def draw_tensors(
             t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * NORM_STD
         elif spec.kind in (VECTOR, CONV):
             t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * VECTOR_STD
+        elif spec.kind == UNIT_INTERVAL:
+            t = 0.05 + 0.9 * torch.rand(spec.shape, generator=gen, dtype=torch.float32, device=device)
+        elif spec.kind == AVERAGE_WEIGHT:
+            n = max(1, spec.shape[-1])
+            t = (1.0 + 0.1 * torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device)) / n
         elif spec.kind == INT_TABLE:
             out[spec.name] = torch.randint(0, 1 << 15, spec.shape, generator=gen, dtype=torch.int32, device=device)
             continue
