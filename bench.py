@@ -82,10 +82,13 @@ def parse() -> argparse.Namespace:
                    help="instead of the decode steps, a case that shapes of one length do not show (prints its own line): "
                         "chunked-prefill: one prompt of --context tokens in portions of --portion tokens; "
                         "mixed-decode: decode steps of --batch - 1 requests of --short tokens beside one of --context tokens")
-    p.add_argument("--design", default=None, choices=["kupuzen", "taborax", "sakevik"],
+    p.add_argument("--design", default=None, choices=["kupuzen", "taborax", "sakevik", "sazilorn"],
                    help="instead of the decode steps: prefill and decode of this design at layer sizes of --design-sizes "
                         "beside the Llama shape of equal width, heads, feed-forward and layers (prints its own line)")
     p.add_argument("--design-sizes", default="1b,3b", help="which sizes of DESIGN_SIZES, comma separated")
+    p.add_argument("--design-beside", default=None, choices=["llama", "kupuzen", "taborax", "sakevik"],
+                   help="the model the --design comparison stands beside (by default the Llama shape; for sazilorn the Kupuzen "
+                        "of equal size, the closest existing design)")
     p.add_argument("--design-only", action="store_true", help="the --design comparison without its Llama half (for profiles)")
     p.add_argument("--design-layers", type=int, default=8, help="layers of both models in the --design comparison")
     p.add_argument("--design-context", type=int, default=4096, help="context at which the --design decode steps end")
@@ -407,24 +410,49 @@ def sakevik_like(size: dict, layers: int) -> dict:
             "logit_scale": 0.5, "layers": [(attention, latent, gru, attention)[i % 4] for i in range(layers)]}
 
 
-DESIGN_MODELS = {"kupuzen": kupuzen_like, "taborax": taborax_like, "sakevik": sakevik_like}
+# A Sazilorn of the same width, vocabulary and number of layers: in every four layers one of HGRN2 (half the Llama heads
+# of twice the size, a dense feed-forward of the Llama inner size), two of soft-capped gated attention (the Llama heads)
+# beside lightning attention (a quarter of the Llama heads of twice the size), one with a mixture whose six chosen
+# experts and shared expert together have the Llama inner size (32 experts) and one dense, and one of attention with
+# a bias by distance (the Llama heads, 32 buckets reaching to 4,096) with a dense feed-forward; a convolution of 4 taps.
+def sazilorn_like(size: dict, layers: int) -> dict:
+    ll = size["llama"]
+    H, G = ll["num_attention_heads"], ll["num_key_value_heads"]
+    d = ll["hidden_size"] // H
+    inner = ll["intermediate_size"]
+    ff = {"kind": "dense", "ff": inner}
+    mixture = {"kind": "moe", "expert": {"ff": inner // 8}, "shared": {"ff": inner // 4}, "router": {"experts": 32, "top": 6, "scale": 2.5}}
+    hgrn2 = {"type": "hgrn2", "mlp": ff, "mixer": {"heads": H // 2, "dim": 2 * d, "vdim": 2 * d}}
+    attention = {"type": "attention", "mlp": ff, "mixer": {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "scale": d ** -0.5,
+                                                           "bias_max": 4096, "bias_buckets": 32}}
+    lightning = {"heads": H // 4, "dim": 2 * d, "vdim": 2 * d, "decay": [1.0 - 2.0 ** -(3 + 7 * i / max(H // 4 - 1, 1)) for i in range(H // 4)]}
+    pair = {"left": {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 50.0}, "right": lightning,
+            "left_scale": 1.0, "right_scale": 0.5}
+    kinds = (hgrn2, {"type": "parallel", "mlp": mixture, "mixer": pair}, attention, {"type": "parallel", "mlp": ff, "mixer": pair})
+    return {"architecture": "Sazilorn", "vocab": ll["vocab_size"], "width": ll["hidden_size"], "max_positions": 32768,
+            "norm": {"eps": 1e-6}, "canon": {"taps": 4}, "layers": [kinds[i % 4] for i in range(layers)]}
+
+
+DESIGN_MODELS = {"kupuzen": kupuzen_like, "taborax": taborax_like, "sakevik": sakevik_like, "sazilorn": sazilorn_like}
 
 
 def run_design(args) -> int:
-    """Prefill of one prompt and decode steps of the new design beside the Llama shape of equal
+    """Prefill of one prompt and decode steps of the new design beside the Llama shape (or another design) of equal
     size, both with seeded random weights through the same runner and engine."""
     import torch
 
-    out = {"metric": f"prefill and decode of {args.design} beside the Llama shape of equal size", "unit": "tokens/s",
+    beside = args.design_beside or ("kupuzen" if args.design == "sazilorn" else "llama")
+    out = {"metric": f"prefill and decode of {args.design} beside the {beside} shape of equal size", "unit": "tokens/s",
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "layers": args.design_layers, "sizes": {}}
     batches = [int(b) for b in args.points.split(",") if b] or [1]
     ctx = args.design_context
     for name in [x for x in args.design_sizes.split(",") if x]:
         size = DESIGN_SIZES[name]
-        configs = {"llama": dict(size["llama"], num_hidden_layers=args.design_layers),
-                   args.design: DESIGN_MODELS[args.design](size, args.design_layers)}
+        other = (dict(size["llama"], num_hidden_layers=args.design_layers) if beside == "llama"
+                 else DESIGN_MODELS[beside](size, args.design_layers))
+        configs = {beside: other, args.design: DESIGN_MODELS[args.design](size, args.design_layers)}
         if args.design_only:
-            del configs["llama"]
+            del configs[beside]
         rec = {}
         for model, cfgd in configs.items():
             runner = build_runner(cfgd, args.dtype, max(batches) * ctx, max(batches), ctx, use_graphs=not args.eager)
@@ -442,7 +470,7 @@ def run_design(args) -> int:
             del runner
             torch.cuda.empty_cache()
         if not args.design_only:
-            rec["ratio"] = {k: round(rec[args.design][k] / rec["llama"][k], 3) for k in rec["llama"] if k.endswith("tok_per_s")}
+            rec["ratio"] = {k: round(rec[args.design][k] / rec[beside][k], 3) for k in rec[beside] if k.endswith("tok_per_s")}
         out["sizes"][name] = rec
     print(json.dumps(out))
     return 0

@@ -82,14 +82,15 @@ def softmax_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: 
     T, H, _ = q.shape
     G = k.shape[1]
     out = torch.zeros((T, H, v.shape[2]), dtype=q.dtype)
+    if rel is not None:
+        by_distance = [distance_bucket(n, rel.shape[0], far) for n in range(T)]
+        idx = torch.tensor([[by_distance[i - j] if j <= i else 0 for j in range(T)] for i in range(T)])
     for h in range(H):
         g = h // (H // G)
         s = (q[:, h] @ k[:, g].T) * scale
         if softcap is not None:
             s = softcap * torch.tanh(s / softcap)
         if rel is not None:
-            B = rel.shape[0]
-            idx = torch.tensor([[distance_bucket(i - j, B, far) if j <= i else 0 for j in range(T)] for i in range(T)])
             s = s + rel[:, h][idx]
         mask = torch.ones((T, T), dtype=torch.bool).tril()
         s = s.masked_fill(~mask, float("-inf"))
@@ -213,7 +214,8 @@ def forward(tokens: list[int], w: dict, cfg: dict, streams: list | None = None) 
     history = [x]
     for i, layer in enumerate(cfg["layers"]):
         h = offset_norm(x, w[f"l{i}.norm1"], eps)
-        mixed = MIXERS[layer["type"]](h + short_convolution(h, w[f"l{i}.canon1"]), w, f"l{i}.mix", layer["mixer"], eps)
+        hm = h + short_convolution(h, w[f"l{i}.canon1"]) if cfg.get("canon") else h
+        mixed = MIXERS[layer["type"]](hm, w, f"l{i}.mix", layer["mixer"], eps)
         ff = feed_forward(h, w, f"l{i}.mlp", layer.get("mlp"))
         history.append(x + (mixed if ff is None else mixed + ff))
         x = depth_average(history, w[f"l{i}.dwa"])

@@ -54,21 +54,45 @@ TK_API int tk_embed_scaled(int dt, const int* ids, const int* last_token, const 
 // more stream that already has the result's rows.  For a norm that reads the result (`nw`, or null) the row
 //     out / sqrt(mean(out^2) + eps) * (offset + nw)
 // is written too, rounded once to T.  One row a workgroup; the sum runs over j in ascending order.
+// `a`, `b` (either may be null): the branches of the block that has just run, with the result's rows; the newest
+// stream (`last`, or the last of `hist` without one) first becomes itself + mult * (a + b), in place: the block's
+// residual sum and this average are one pass.
 // --------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void depth_average_kernel(const float* __restrict__ hist, size_t stride, int count,
-                                                            const float* __restrict__ last, const int* __restrict__ rows,
+__global__ __launch_bounds__(256) void depth_average_kernel(float* __restrict__ hist, size_t stride, int count,
+                                                            float* __restrict__ last, const int* __restrict__ rows,
                                                             const float* __restrict__ w, float* __restrict__ out,
                                                             const float* __restrict__ nw, float offset, float eps,
-                                                            T* __restrict__ normed, int hidden) {
+                                                            T* __restrict__ normed, int hidden, const float* __restrict__ a,
+                                                            const float* __restrict__ b, float mult) {
   __shared__ float red[16];
   const size_t r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : r;
+  const bool pending = a || b;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float branch = 0.f;
+    if (pending) {
+      branch = a ? a[r * hidden + i] : 0.f;
+      if (b) branch += b[r * hidden + i];
+    }
     float acc = 0.f;
-    for (int j = 0; j < count; ++j) acc = fmaf(w[j], hist[(size_t)j * stride + src * hidden + i], acc);
-    if (last) acc = fmaf(w[count], last[r * hidden + i], acc);
+    for (int j = 0; j < count; ++j) {
+      float v = hist[(size_t)j * stride + src * hidden + i];
+      if (pending && !last && j == count - 1) {
+        v = fmaf(mult, branch, v);
+        hist[(size_t)j * stride + src * hidden + i] = v;
+      }
+      acc = fmaf(w[j], v, acc);
+    }
+    if (last) {
+      float v = last[r * hidden + i];
+      if (pending) {
+        v = fmaf(mult, branch, v);
+        last[r * hidden + i] = v;
+      }
+      acc = fmaf(w[count], v, acc);
+    }
     out[r * hidden + i] = acc;
     ss = fmaf(acc, acc, ss);
   }
@@ -79,19 +103,20 @@ __global__ __launch_bounds__(256) void depth_average_kernel(const float* __restr
     normed[r * hidden + i] = from_f32<T>(out[r * hidden + i] * rstd * (offset + nw[i]));
 }
 
-TK_API int tk_depth_average(int dt, const float* hist, size_t stride, int count, const float* last, const int* rows,
+TK_API int tk_depth_average(int dt, float* hist, size_t stride, int count, float* last, const int* rows,
                             const float* w, float* out, const float* nw, float offset, float eps, void* normed,
-                            int n_rows, int hidden, hipStream_t stream) {
+                            int n_rows, int hidden, const float* a, const float* b, float mult, hipStream_t stream) {
+  TK_REQUIRE(!(a || b) || last || !rows, "depth_average: branches are added to a stream that has the result's rows");
   TK_REQUIRE(n_rows >= 0 && hidden > 0 && count >= 0 && (count > 0 || last) && w && out && (count == 0 || hist),
              "depth_average: bad sizes rows=%d hidden=%d streams=%d or a pointer is missing", n_rows, hidden, count);
   TK_REQUIRE(!nw || normed, "depth_average: a norm's weight needs a place for its rows");
   if (n_rows == 0) return 0;
   if (dt == TK_F32)
     hipLaunchKernelGGL(depth_average_kernel<float>, dim3(n_rows), dim3(256), 0, stream, hist, stride, count, last, rows, w, out,
-                       nw, offset, eps, (float*)normed, hidden);
+                       nw, offset, eps, (float*)normed, hidden, a, b, mult);
   else
     hipLaunchKernelGGL(depth_average_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, stream, hist, stride, count, last, rows, w, out,
-                       nw, offset, eps, (bf16_t*)normed, hidden);
+                       nw, offset, eps, (bf16_t*)normed, hidden, a, b, mult);
   TK_CHECK_LAUNCH("depth_average");
   return 0;
 }

@@ -1183,15 +1183,19 @@ def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, last_toke
 
 def depth_average(hist: torch.Tensor, count: int, weights: torch.Tensor, last: torch.Tensor | None = None,
                   rows: torch.Tensor | None = None, out: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None,
-                  unit_offset: bool = False, eps: float = 0.0, out_dtype: torch.dtype = torch.float32
+                  unit_offset: bool = False, eps: float = 0.0, out_dtype: torch.dtype = torch.float32,
+                  branches: tuple[torch.Tensor | None, torch.Tensor | None] = (None, None), mult: float = 1.0
                   ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """A weighted sum over the streams a model has had so far: ``hist`` [streams, tokens, H] (32-bit) of which the
     first ``count`` count, ``weights`` (32-bit, one number a stream, ``last``'s behind the others); ``rows`` (int32):
     only these rows of the streams are wanted, in this order; ``last`` [len(rows) or tokens, H]: one more stream that
     already has the result's rows.  ``out``: where the result goes (a contiguous 32-bit buffer of its shape).
     ``norm_weight`` (32-bit [H]): also returns the result's rows through an RMS norm with this weight (plus one
-    with ``unit_offset``), rounded once to ``out_dtype``."""
-    _gpu(hist, weights, last, rows, out, norm_weight)
+    with ``unit_offset``), rounded once to ``out_dtype``.  ``branches`` (32-bit, the result's shape; either may be
+    None): the newest stream (``last``, or the last counted of ``hist``) first becomes itself + ``mult`` * (a + b), in
+    place: a block's residual sum in the same pass."""
+    a, b = branches
+    _gpu(hist, weights, last, rows, out, norm_weight, a, b)
     _need(hist.dim() == 3 and hist.dtype == torch.float32 and hist.is_contiguous() and 0 <= count <= hist.shape[0],
           "depth_average: the streams must be contiguous float32 [streams, tokens, H]")
     hidden = hist.shape[2]
@@ -1203,6 +1207,11 @@ def depth_average(hist: torch.Tensor, count: int, weights: torch.Tensor, last: t
     _need(rows is not None or n == hist.shape[1], "depth_average: without chosen rows every stream has the result's rows")
     _f32_vector(weights, count + (1 if last is not None else 0), "depth_average: the weights")
     _f32_vector(norm_weight, hidden, "depth_average: a norm weight")
+    for y in (a, b):
+        _need(y is None or (y.shape == (n, hidden) and y.dtype == torch.float32 and y.is_contiguous()),
+              "depth_average: a branch must be contiguous float32 of the result's shape")
+    _need((a is None and b is None) or last is not None or (rows is None and count > 0),
+          "depth_average: branches are added to a stream that has the result's rows")
     if out is None:
         out = torch.empty((n, hidden), dtype=torch.float32, device=hist.device)
     _need(out.shape == (n, hidden) and out.dtype == torch.float32 and out.is_contiguous(), "depth_average: the result's buffer")
@@ -1211,7 +1220,8 @@ def depth_average(hist: torch.Tensor, count: int, weights: torch.Tensor, last: t
         call("tk_depth_average", dtype_code(out_dtype), hist.data_ptr(), hist.stride(0), int(count),
              last.data_ptr() if last is not None else None, rows.data_ptr() if rows is not None else None, weights.data_ptr(),
              out.data_ptr(), norm_weight.data_ptr() if norm_weight is not None else None, 1.0 if unit_offset else 0.0, float(eps),
-             normed.data_ptr() if normed is not None else None, n, hidden, _stream())
+             normed.data_ptr() if normed is not None else None, n, hidden, a.data_ptr() if a is not None else None,
+             b.data_ptr() if b is not None else None, float(mult), _stream())
     return out, normed
 
 

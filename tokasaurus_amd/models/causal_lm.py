@@ -112,7 +112,13 @@ class CausalLM:
                 reader = self.head.entry_norm()
             elif order[i + 1].before is None:  # (else the stream changes before the next block reads it)
                 reader = self.blocks[order[i + 1].layer].entry_norm()
-            if block.fuses_norm:
+            after = self.connectors[entry.after] if entry.after is not None else None
+            pending = None
+            if block.fuses_norm and after is not None and getattr(after, "adds_pending_sum", False) and getattr(block, "can_defer_sum", False):
+                # the block hands its branches over unsummed: the connector behind it adds them in its own pass
+                pending = block.forward(x, ctx, caches[i], states[i], rows, prepared=prepared, next_norm=None, defer_sum=True)
+                out = pending.x
+            elif block.fuses_norm:
                 # (a connector behind this block changes the stream before anything reads it)
                 out = block.forward(x, ctx, caches[i], states[i], rows, prepared=prepared,
                                     next_norm=None if entry.after is not None else reader)
@@ -123,10 +129,10 @@ class CausalLM:
                 whole = rows is None
                 if whole and x.data_ptr() != hist[i + 1].data_ptr():
                     hist[i + 1].copy_(x)  # (a block that did not update its input in place)
-                after = self.connectors[entry.after] if entry.after is not None else None
                 if after is not None and getattr(after, "takes_history", False):
+                    more = {"pending": pending} if pending is not None else {}
                     out = after.forward_history(hist, i + 2 if whole else i + 1, None if whole else x, rows,
-                                                hist[i + 2] if (whole and i < last) else None, next_norm=reader)
+                                                hist[i + 2] if (whole and i < last) else None, next_norm=reader, **more)
                     x, prepared = stream_and_prepared(out)
                 elif i < last:
                     hist[i + 2].copy_(x)

@@ -122,6 +122,14 @@ class NormPair(Part):
         return h1, h2
 
 
+class PendingSum:
+    """A block's residual sum that has not been made: ``x + mult * (a + b)`` with ``x`` the block's input rows
+    (the wanted rows only, for a step's last block) and the branches' 32-bit sums (either may be None)."""
+
+    def __init__(self, x: torch.Tensor, branches: tuple, mult: float):
+        self.x, self.branches, self.mult = x, branches, float(mult)
+
+
 @BLOCKS.register("parallel_residual")
 class ParallelResidualBlock(Block):
     """Mixer and feed-forward side by side on a 32-bit residual stream:
@@ -173,7 +181,12 @@ class ParallelResidualBlock(Block):
     def entry_norm(self):
         return self.entry
 
-    def forward(self, x, ctx: StepContext, cache, state, rows, prepared: Prepared | None = None, next_norm=None):
+    can_defer_sum = True
+
+    def forward(self, x, ctx: StepContext, cache, state, rows, prepared: Prepared | None = None, next_norm=None,
+                defer_sum: bool = False):
+        """``defer_sum``: the stream is not updated; returns ``PendingSum`` (the block's input rows, its branches and
+        the multiplier) for whoever runs next on the stream and can add them in its own pass."""
         if x.dtype != torch.float32:
             raise TypeError("a parallel_residual block runs on a 32-bit stream (an embedding with stream_f32)")
         if prepared is not None and prepared.norm is self.entry and prepared.normed is not None:
@@ -195,6 +208,8 @@ class ParallelResidualBlock(Block):
             x = ops.gather_rows(x, rows)
             h2 = ops.gather_rows(h2, rows) if h2 is not None else None
         b = self.feed_forward.transform(h2, out_f32=True) if self.feed_forward is not None else None
+        if defer_sum:
+            return PendingSum(x, (a, b), self.residual_mult)
         # the norms that read the new stream: the next block's pair or a single norm (the head's)
         first = second = None
         if isinstance(next_norm, NormPair) and next_norm.fused():
@@ -387,6 +402,7 @@ class DepthAverage(Connector):
     pass writes that norm's rows."""
 
     takes_history = True
+    adds_pending_sum = True  # a block in front may hand over its branches unsummed (``PendingSum``)
 
     def __init__(self, streams: int, name: str):
         self.streams, self.name = int(streams), name
@@ -399,9 +415,10 @@ class DepthAverage(Connector):
         self.weight = placer.place(("vector_f32", self.name), lambda: tensors[self.name].to(torch.float32).contiguous().to(placer.device))
 
     def forward_history(self, hist: torch.Tensor, count: int, last: torch.Tensor | None, rows: torch.Tensor | None,
-                        out: torch.Tensor | None, next_norm=None):
+                        out: torch.Tensor | None, next_norm=None, pending: "PendingSum | None" = None):
         """``hist`` [streams, tokens, H]: X_0 .. X_(count - 1); ``last``: X_count where it has only the wanted
-        ``rows``.  Returns the new stream (in ``out`` when given), or (stream, ``Prepared``) for ``next_norm``."""
+        ``rows``.  ``pending``: the newest of these is still the block's input and becomes its result here.
+        Returns the new stream (in ``out`` when given), or (stream, ``Prepared``) for ``next_norm``."""
         if count + (1 if last is not None else 0) != self.streams:
             raise RuntimeError(f"a depth average over {self.streams} streams was handed {count + (1 if last is not None else 0)}")
         reader = next_norm.first if isinstance(next_norm, NormPair) and next_norm.second is None else next_norm
@@ -411,7 +428,9 @@ class DepthAverage(Connector):
                                       norm_weight=reader.weight if reader is not None else None,
                                       unit_offset=reader.unit_offset if reader is not None else False,
                                       eps=reader.eps if reader is not None else 0.0,
-                                      out_dtype=reader.out_dtype if reader is not None else torch.float32)
+                                      out_dtype=reader.out_dtype if reader is not None else torch.float32,
+                                      branches=pending.branches if pending is not None else (None, None),
+                                      mult=pending.mult if pending is not None else 1.0)
         if reader is None:
             return x
         return x, Prepared(None, next_norm, (normed, None) if isinstance(next_norm, NormPair) else normed)
