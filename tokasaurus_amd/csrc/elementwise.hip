@@ -315,15 +315,39 @@ __global__ void gelu_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   if (i < inter) out[(size_t)blockIdx.y * inter + i] = from_f32<T>(gelu_tanh_f32(to_f32<T>(g[i])) * to_f32<T>(u[i]));
 }
 
+// (16 bytes a load where sizes and addresses allow)
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_glu_packed_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+  constexpr int N = Pack<T>::N;
+  const int piece = blockIdx.x * blockDim.x + threadIdx.x;
+  if (piece >= inter / N) return;
+  const T* g = gu + (size_t)blockIdx.y * 2 * inter + (size_t)piece * N;
+  Pack<T> gv, uv, o;
+  gv.load(g);
+  uv.load(g + inter);
+#pragma unroll
+  for (int j = 0; j < N; ++j) o.v[j] = from_f32<T>(gelu_tanh_f32(to_f32<T>(gv.v[j])) * to_f32<T>(uv.v[j]));
+  o.store(out + (size_t)blockIdx.y * inter + (size_t)piece * N);
+}
+
+template <typename T>
+static void launch_gelu_glu(const void* gate_up, void* out, int rows, int inter, hipStream_t stream) {
+  constexpr int N = Pack<T>::N;
+  if (inter % N == 0 && aligned16(gate_up) && aligned16(out))
+    hipLaunchKernelGGL(gelu_glu_packed_kernel<T>, dim3((inter / N + 255) / 256, rows), dim3(256), 0, stream, (const T*)gate_up,
+                       (T*)out, inter);
+  else
+    hipLaunchKernelGGL(gelu_glu_kernel<T>, dim3((inter + 255) / 256, rows), dim3(256), 0, stream, (const T*)gate_up, (T*)out, inter);
+}
+
 TK_API int tk_gelu_glu(int dt, const void* gate_up, void* out, int rows, int inter, hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && inter > 0, "gelu_glu: bad sizes %d %d", rows, inter);
   TK_REQUIRE(rows < 65536, "gelu_glu: %d rows are too many for one call", rows);
   if (rows == 0) return 0;
-  const dim3 grid((inter + 255) / 256, rows);
   if (dt == TK_F32)
-    hipLaunchKernelGGL(gelu_glu_kernel<float>, grid, dim3(256), 0, stream, (const float*)gate_up, (float*)out, inter);
+    launch_gelu_glu<float>(gate_up, out, rows, inter, stream);
   else
-    hipLaunchKernelGGL(gelu_glu_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)gate_up, (bf16_t*)out, inter);
+    launch_gelu_glu<bf16_t>(gate_up, out, rows, inter, stream);
   TK_CHECK_LAUNCH("gelu_glu");
   return 0;
 }

@@ -11,128 +11,185 @@
 // Everything from the sums on (activations, gates, the state, the read-out) is 32-bit arithmetic.
 //
 // The state row of a slot is [H][dv][dk]: a value column's dk numbers lie together.  The columns of S
-// do not meet: a column is owned by LA_LANES neighbouring lanes that cut dk between them (lane l holds rows
-// l + LA_LANES * n) and add up through the wavefront's own data paths, always in the same order, so a
-// token's result does not depend on how its request's tokens were cut into steps or on what shares the batch.
+// do not meet: a column is owned by LA_LANES neighbouring lanes that cut dk between them and add up through the
+// wavefront's own data paths, always in the same order, so a token's result does not depend on how its request's
+// tokens were cut into steps or on what shares the batch.
 #include "common.h"
 
 #define LA_LANES 16
-#define LA_COLS 16     // value columns a workgroup owns (LA_COLS * LA_LANES threads)
-#define LA_TOKENS 16   // tokens staged in LDS at a time
+#define LA_COLS 4      // value columns a wavefront owns; a workgroup is one wavefront
 enum { LA_CONSTANT = 0, LA_FORGET = 1 };
 
 __device__ __forceinline__ float la_silu(float x) { return x / (1.0f + expf(-x)); }
 __device__ __forceinline__ float la_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-// Workgroup (head, request, block of LA_COLS value columns).  A chunk of tokens is staged as
-// [tokens][q | k | a (dkp each)][v (LA_COLS)], activations applied on the way in.
-template <int NQ, int MODE>
-__global__ __launch_bounds__(LA_COLS * LA_LANES) void linear_attention_kernel(
-    const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
-    const float* __restrict__ f_bias, const float* __restrict__ f_low, float* __restrict__ state, size_t state_stride,
-    const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ o, int H, int dk, int dv) {
-  constexpr int dkp = NQ * LA_LANES;
-  constexpr int row_floats = 3 * dkp + LA_COLS;
-  __shared__ float stage[LA_TOKENS * row_floats];
+// --------------------------------------------------------------------------
+// Before the recurrence, once a token: the activations, into rows that the recurrence's lanes read 16 bytes at a
+// time.  rec row: [q: H x dkp | k or f: H x dkp | v: H x dv (padded to a multiple of 4)], dkp = dk rounded up to a
+// multiple of 64, zeros in the padding (a padded row of S meets a zero of q).
+//   LA_CONSTANT  q = silu(.), k = silu(.), v = silu(.)
+//   LA_FORGET    q = silu(.), f = low + (1 - low) * sigmoid(. + bias), v as it is
+// --------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(256) void linear_attention_prepare_kernel(
+    const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, const float* __restrict__ f_bias,
+    const float* __restrict__ f_low, float* __restrict__ rec, int ld_rec, int H, int dk, int dv, int dkp) {
+  const size_t t = blockIdx.y;
+  const int x = blockIdx.x * blockDim.x + threadIdx.x;
+  if (x >= ld_rec) return;
+  const float* row = proj + t * ld;
+  float val = 0.f;
+  if (x < 2 * H * dkp) {
+    const int which = x / (H * dkp), rem = x % (H * dkp), h = rem / dkp, i = rem % dkp;
+    if (i < dk) {
+      const int c = h * dk + i;
+      if (which == 0) {
+        val = la_silu(row[q_off + c]);
+      } else if (MODE == LA_CONSTANT) {
+        val = la_silu(row[k_off + c]);
+      } else {
+        const float lo = f_low[c];
+        val = lo + (1.0f - lo) * la_sigmoid(row[k_off + c] + f_bias[c]);
+      }
+    }
+  } else {
+    const int c = x - 2 * H * dkp;
+    if (c < H * dv) val = MODE == LA_CONSTANT ? la_silu(row[v_off + c]) : row[v_off + c];
+  }
+  rec[t * ld_rec + x] = val;
+}
+
+// --------------------------------------------------------------------------
+// The recurrence.  A workgroup is one wavefront: (head, request, block of LA_COLS value columns).  A column of S is
+// owned by LA_LANES neighbouring lanes; lane l holds rows 4 * (l + LA_LANES * n) + e, n < NQ, e < 4, so that it reads
+// its pieces of q and of k (or f) as whole 16-byte loads.  Nothing is staged in LDS and there is no barrier: the
+// wavefronts of a head read the same rows of `rec` (served by the caches), PF tokens ahead of the arithmetic.
+//   LA_CONSTANT  s = a s + k v        LA_FORGET  s = f s + (1 - f) v = v + f (s - v)        o = sum over rows of q s
+// --------------------------------------------------------------------------
+template <int NQ, int MODE, int PF>
+__global__ __launch_bounds__(TK_WAVE) void linear_attention_kernel(
+    const float* __restrict__ rec, int ld_rec, const float* __restrict__ decay, float* __restrict__ state,
+    size_t state_stride, const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ o, int H,
+    int dk, int dv, int dkp) {
   const int h = blockIdx.x, r = blockIdx.y;
-  const int col0 = blockIdx.z * LA_COLS;
   const int lane = threadIdx.x % LA_LANES, grp = threadIdx.x / LA_LANES;
-  const int col = col0 + grp;
+  const int col = blockIdx.z * LA_COLS + grp;
   const bool live = col < dv;
   const int first = q_start[r], last = q_start[r + 1];
+  if (first >= last) return;
   float* s_col = state + (size_t)slots[r] * state_stride + ((size_t)h * dv + (live ? col : 0)) * dk;
-  float s[NQ];
+  const bool vec = (dk % 4 == 0) && (state_stride % 4 == 0);
+  float s[NQ][4];
 #pragma unroll
   for (int n = 0; n < NQ; ++n) {
-    const int i = lane + LA_LANES * n;
-    s[n] = (live && i < dk) ? s_col[i] : 0.f;
+    const int i = 4 * (lane + LA_LANES * n);
+    if (vec && live && i < dk) {
+      const float4 v = *(const float4*)(s_col + i);
+      s[n][0] = v.x; s[n][1] = v.y; s[n][2] = v.z; s[n][3] = v.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[n][e] = (live && i + e < dk) ? s_col[i + e] : 0.f;
+    }
   }
   const float a_head = MODE == LA_CONSTANT ? decay[h] : 0.f;
-#pragma unroll 1
-  for (int t0 = first; t0 < last; t0 += LA_TOKENS) {
-    const int nt = min(LA_TOKENS, last - t0);
-    __syncthreads();  // the chunk before is consumed
-    for (int x = threadIdx.x; x < nt * row_floats; x += blockDim.x) {
-      const int tt = x / row_floats, rem = x % row_floats;
-      const float* row = proj + (size_t)(t0 + tt) * ld;
-      float val = 0.f;
-      if (rem < 3 * dkp) {
-        const int which = rem / dkp, i = rem % dkp;
-        if (i < dk) {
-          const int c = h * dk + i;
-          if (MODE == LA_CONSTANT) {
-            val = which == 0 ? la_silu(row[q_off + c]) : (which == 1 ? la_silu(row[k_off + c]) : a_head);
-          } else {
-            if (which == 0) {
-              val = la_silu(row[q_off + c]);
-            } else {
-              const float lo = f_low[c];
-              const float f = lo + (1.0f - lo) * la_sigmoid(row[k_off + c] + f_bias[c]);
-              val = which == 1 ? 1.0f - f : f;
-            }
-          }
-        }
-      } else {
-        const int c = col0 + rem - 3 * dkp;
-        if (c < dv) {
-          const float v = row[v_off + h * dv + c];
-          val = MODE == LA_CONSTANT ? la_silu(v) : v;
-        }
-      }
-      stage[x] = val;
-    }
-    __syncthreads();
-#pragma unroll 1
-    for (int tt = 0; tt < nt; ++tt) {
-      const float* row = stage + tt * row_floats;
-      const float v = row[3 * dkp + grp];
-      float acc = 0.f;
-#pragma unroll
-      for (int n = 0; n < NQ; ++n) {
-        const int i = lane + LA_LANES * n;
-        s[n] = fmaf(row[2 * dkp + i], s[n], row[dkp + i] * v);
-        acc = fmaf(row[i], s[n], acc);
-      }
-      acc = row_sum16(acc);
-      if (live && lane == 0) o[(size_t)(t0 + tt) * H * dv + (size_t)h * dv + col] = acc;
-    }
+  const int q_at = h * dkp + 4 * lane, k_at = H * dkp + q_at, v_at = 2 * H * dkp + h * dv + (live ? col : 0);
+
+  float4 q[2][PF][NQ], k[2][PF][NQ];
+  float v[2][PF];
+  // rows of tokens t0 .. t0 + PF - 1 (those beyond the request's end repeat its last token and are not used)
+#define LA_LOAD(B, T0)                                                               \
+  _Pragma("unroll") for (int j = 0; j < PF; ++j) {                                   \
+    const float* row = rec + (size_t)min((T0) + j, last - 1) * ld_rec;               \
+    _Pragma("unroll") for (int n = 0; n < NQ; ++n) {                                 \
+      q[B][j][n] = *(const float4*)(row + q_at + 4 * LA_LANES * n);                  \
+      k[B][j][n] = *(const float4*)(row + k_at + 4 * LA_LANES * n);                  \
+    }                                                                                \
+    v[B][j] = row[v_at];                                                             \
   }
-  if (live) {
+#define LA_STEP(B, T0)                                                               \
+  _Pragma("unroll") for (int j = 0; j < PF; ++j) {                                   \
+    if ((T0) + j < last) {                                                           \
+      const float vv = v[B][j];                                                      \
+      float acc0 = 0.f, acc1 = 0.f;                                                  \
+      _Pragma("unroll") for (int n = 0; n < NQ; ++n) {                               \
+        const float qq[4] = {q[B][j][n].x, q[B][j][n].y, q[B][j][n].z, q[B][j][n].w}; \
+        const float kk[4] = {k[B][j][n].x, k[B][j][n].y, k[B][j][n].z, k[B][j][n].w}; \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) {                              \
+          if (MODE == LA_CONSTANT) s[n][e] = fmaf(a_head, s[n][e], kk[e] * vv);      \
+          else s[n][e] = fmaf(kk[e], s[n][e] - vv, vv);                              \
+        }                                                                            \
+        acc0 = fmaf(qq[0], s[n][0], acc0); acc1 = fmaf(qq[1], s[n][1], acc1);        \
+        acc0 = fmaf(qq[2], s[n][2], acc0); acc1 = fmaf(qq[3], s[n][3], acc1);        \
+      }                                                                              \
+      const float sum = row_sum16(acc0 + acc1);                                      \
+      if (live && lane == 0) o[(size_t)((T0) + j) * H * dv + (size_t)h * dv + col] = sum; \
+    }                                                                                \
+  }
+  LA_LOAD(0, first);
+#pragma unroll 1
+  for (int t0 = first; t0 < last; t0 += 2 * PF) {
+    LA_LOAD(1, t0 + PF);
+    LA_STEP(0, t0);
+    LA_LOAD(0, t0 + 2 * PF);
+    LA_STEP(1, t0 + PF);
+  }
+#undef LA_LOAD
+#undef LA_STEP
 #pragma unroll
-    for (int n = 0; n < NQ; ++n) {
-      const int i = lane + LA_LANES * n;
-      if (i < dk) s_col[i] = s[n];
+  for (int n = 0; n < NQ; ++n) {
+    const int i = 4 * (lane + LA_LANES * n);
+    if (!live) continue;
+    if (vec && i < dk) {
+      *(float4*)(s_col + i) = make_float4(s[n][0], s[n][1], s[n][2], s[n][3]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (i + e < dk) s_col[i + e] = s[n][e];
     }
   }
 }
 
+// Floats of a row of `rec` for these sizes, and the padded size of a head's keys.
+TK_API int tk_linear_attention_rec_width(int H, int dk, int dv) {
+  const int dkp = (dk + 63) / 64 * 64;
+  return 2 * H * dkp + (H * dv + 3) / 4 * 4;
+}
+
 TK_API int tk_linear_attention(int mode, const float* proj, int ld, int q_off, int k_off, int v_off, const float* decay,
                                const float* f_bias, const float* f_low, float* state, size_t state_stride,
-                               const int* q_start, const int* slots, float* o, int n_requests, int H, int dk, int dv,
-                               hipStream_t stream) {
-  TK_REQUIRE(n_requests >= 0 && H > 0 && dk > 0 && dv > 0 && dk <= 16 * LA_LANES,
-             "linear_attention: bad sizes requests=%d heads=%d dk=%d dv=%d (dk up to %d)", n_requests, H, dk, dv, 16 * LA_LANES);
+                               const int* q_start, const int* slots, float* rec, float* o, int n_tokens, int n_requests, int H,
+                               int dk, int dv, hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && n_requests >= 0 && H > 0 && dk > 0 && dv > 0 && dk <= 256,
+             "linear_attention: bad sizes tokens=%d requests=%d heads=%d dk=%d dv=%d (dk up to 256)", n_tokens, n_requests, H, dk, dv);
   TK_REQUIRE(mode == LA_CONSTANT ? decay != nullptr : (mode == LA_FORGET && f_bias && f_low),
              "linear_attention: the constant form needs a decay a head, the forget-gate form a bias and a lower bound");
-  TK_REQUIRE(proj && state && q_start && slots && o && state_stride >= (size_t)H * dk * dv && n_requests < 65536,
-             "linear_attention: a pointer is missing, the state's rows are too short or the requests too many");
-  if (n_requests == 0) return 0;
-  const int nq = (dk + LA_LANES - 1) / LA_LANES;
-  const dim3 grid(H, n_requests, (dv + LA_COLS - 1) / LA_COLS), block(LA_COLS * LA_LANES);
-#define LA_CASE(NQ)                                                                                                              \
-  do {                                                                                                                           \
-    if (mode == LA_CONSTANT)                                                                                                     \
-      hipLaunchKernelGGL((linear_attention_kernel<NQ, LA_CONSTANT>), grid, block, 0, stream, proj, ld, q_off, k_off, v_off,      \
-                         decay, f_bias, f_low, state, state_stride, q_start, slots, o, H, dk, dv);                               \
-    else                                                                                                                         \
-      hipLaunchKernelGGL((linear_attention_kernel<NQ, LA_FORGET>), grid, block, 0, stream, proj, ld, q_off, k_off, v_off, decay, \
-                         f_bias, f_low, state, state_stride, q_start, slots, o, H, dk, dv);                                      \
+  TK_REQUIRE(proj && state && q_start && slots && o && rec && state_stride >= (size_t)H * dk * dv && n_requests < 65536 && n_tokens < 65536,
+             "linear_attention: a pointer is missing, the state's rows are too short or the step too large");
+  TK_REQUIRE((((uintptr_t)rec | (uintptr_t)state) & 15) == 0, "linear_attention: rec and state must start at multiples of 16 bytes");
+  if (n_requests == 0 || n_tokens == 0) return 0;
+  const int dkp = (dk + 63) / 64 * 64, nq = dkp / 64;
+  const int ld_rec = tk_linear_attention_rec_width(H, dk, dv);
+  const dim3 pgrid((ld_rec + 255) / 256, n_tokens);
+  if (mode == LA_CONSTANT)
+    hipLaunchKernelGGL(linear_attention_prepare_kernel<LA_CONSTANT>, pgrid, dim3(256), 0, stream, proj, ld, q_off, k_off, v_off,
+                       f_bias, f_low, rec, ld_rec, H, dk, dv, dkp);
+  else
+    hipLaunchKernelGGL(linear_attention_prepare_kernel<LA_FORGET>, pgrid, dim3(256), 0, stream, proj, ld, q_off, k_off, v_off,
+                       f_bias, f_low, rec, ld_rec, H, dk, dv, dkp);
+  const dim3 grid(H, n_requests, (dv + LA_COLS - 1) / LA_COLS), block(TK_WAVE);
+#define LA_CASE(NQ, PF)                                                                                                      \
+  do {                                                                                                                       \
+    if (mode == LA_CONSTANT)                                                                                                 \
+      hipLaunchKernelGGL((linear_attention_kernel<NQ, LA_CONSTANT, PF>), grid, block, 0, stream, rec, ld_rec, decay, state,  \
+                         state_stride, q_start, slots, o, H, dk, dv, dkp);                                                   \
+    else                                                                                                                     \
+      hipLaunchKernelGGL((linear_attention_kernel<NQ, LA_FORGET, PF>), grid, block, 0, stream, rec, ld_rec, decay, state,    \
+                         state_stride, q_start, slots, o, H, dk, dv, dkp);                                                   \
   } while (0)
-  if (nq <= 1) LA_CASE(1);
-  else if (nq <= 2) LA_CASE(2);
-  else if (nq <= 4) LA_CASE(4);
-  else if (nq <= 8) LA_CASE(8);
-  else LA_CASE(16);
+  if (nq <= 1) LA_CASE(1, 4);
+  else if (nq <= 2) LA_CASE(2, 4);
+  else if (nq <= 3) LA_CASE(3, 2);
+  else LA_CASE(4, 2);
 #undef LA_CASE
   TK_CHECK_LAUNCH("linear_attention");
   return 0;

@@ -1255,12 +1255,15 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, sta
     _f32_vector(decay, H, "linear_attention: the decays")
     _f32_vector(forget_bias, H * dk, "linear_attention: the forget gate's bias")
     _f32_vector(forget_low, H * dk, "linear_attention: the forget gate's lower bound")
+    _need(dk <= 256, f"linear_attention: heads of up to 256 key channels, not {dk}")
     o = torch.empty((n, H * dv), dtype=torch.float32, device=proj.device)
     if n:
+        # the activated rows that the recurrence reads: one pass over the step's tokens in front of it
+        rec = torch.empty((n, load("core").tk_linear_attention_rec_width(H, dk, dv)), dtype=torch.float32, device=proj.device)
         call("tk_linear_attention", 0 if constant else 1, proj.data_ptr(), proj.stride(0), int(q_off), int(k_off), int(v_off),
              decay.data_ptr() if constant else None, forget_bias.data_ptr() if not constant else None,
              forget_low.data_ptr() if not constant else None, state.data_ptr(), state.stride(0), q_start.data_ptr(),
-             slots.data_ptr(), o.data_ptr(), slots.numel(), H, dk, dv, _stream())
+             slots.data_ptr(), rec.data_ptr(), o.data_ptr(), n, slots.numel(), H, dk, dv, _stream())
     return o
 
 
