@@ -135,22 +135,36 @@ def test_short_convolution_kernel(dtype, width, taps, lens):
             at += ln
 
 
-def test_depth_average_kernel():
-    """The weighted sum over the streams so far, with and without a last stream that has only the wanted rows, and
-    the norm's rows from the same pass."""
+@pytest.mark.parametrize("width", [70, 256, 1028])
+def test_depth_average_kernel(width):
+    """The weighted sum over the streams so far, with and without a last stream that has only the wanted rows, the
+    norm's rows from the same pass, and a block's branches added to the newest stream on the way."""
     torch.manual_seed(3)
-    hist = torch.randn(5, 9, 70).cuda()
+    hist = torch.randn(5, 9, width).cuda()
     w = torch.randn(4).cuda()
-    nw = torch.randn(70).cuda() * 0.1
+    nw = torch.randn(width).cuda() * 0.1
     out, normed = ops.depth_average(hist, 4, w, norm_weight=nw, unit_offset=True, eps=1e-5, out_dtype=torch.float32)
     want = sum(w[j].double().cpu() * hist[j].double().cpu() for j in range(4))
     assert torch.allclose(out.cpu().double(), want, atol=1e-5)
     assert torch.allclose(normed.cpu().double(), pz.offset_norm(want, nw.cpu().double(), 1e-5), atol=1e-5)
     rows = torch.tensor([8, 0, 3], dtype=torch.int32).cuda()
-    last = torch.randn(3, 70).cuda()
+    last = torch.randn(3, width).cuda()
     out, normed = ops.depth_average(hist, 3, w, last=last, rows=rows, out_dtype=torch.bfloat16)
     want = sum(w[j].double().cpu() * hist[j].double().cpu()[[8, 0, 3]] for j in range(3)) + w[3].double().cpu() * last.double().cpu()
     assert normed is None and torch.allclose(out.cpu().double(), want, atol=1e-5)
+    # branches: the newest stream becomes itself + mult * (a + b), in place, before it is weighed
+    a, b = torch.randn(9, width).cuda(), torch.randn(9, width).cuda()
+    h2 = hist.clone()
+    out, _ = ops.depth_average(h2, 4, w, branches=(a, b), mult=0.5)
+    newest = hist[3].double().cpu() + 0.5 * (a.double().cpu() + b.double().cpu())
+    want = sum(w[j].double().cpu() * hist[j].double().cpu() for j in range(3)) + w[3].double().cpu() * newest
+    assert torch.allclose(out.cpu().double(), want, atol=1e-5) and torch.allclose(h2[3].cpu().double(), newest, atol=1e-6)
+    assert torch.equal(h2[:3], hist[:3]) and torch.equal(h2[4], hist[4])
+    l2 = last.clone()
+    out, _ = ops.depth_average(hist, 3, w, last=l2, rows=rows, branches=(a[:3].contiguous(), None), mult=2.0)
+    newest = last.double().cpu() + 2.0 * a[:3].double().cpu()
+    want = sum(w[j].double().cpu() * hist[j].double().cpu()[[8, 0, 3]] for j in range(3)) + w[3].double().cpu() * newest
+    assert torch.allclose(out.cpu().double(), want, atol=1e-5) and torch.allclose(l2.cpu().double(), newest, atol=1e-6)
 
 
 def test_router_with_normalised_weights():

@@ -40,7 +40,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
         "tk_embed_scaled": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, _P, c_int, _P],
         "tk_depth_average": [c_int, _P, c_size_t, c_int, _P, _P, _P, _P, _P, c_float, c_float, _P, c_int, c_int, _P, _P, c_float, _P],
-        "tk_linear_attention": [c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, c_size_t, _P, _P, _P, _P] + [c_int] * 5 + [_P],
+        "tk_linear_attention": [c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, c_size_t, _P, _P, _P, _P] + [c_int] * 6 + [_P],
         "tk_linear_attention_rec_width": [c_int, c_int, c_int],
         "tk_group_norm_gate": [c_int, _P, _P, c_int, _P, c_float, c_float, _P, c_int, c_int, c_int, c_int, _P],
         "tk_sigmoid_gate": [c_int, _P, c_int, _P, c_int, c_float, _P, c_int, c_int, c_int, _P],

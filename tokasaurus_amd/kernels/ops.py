@@ -1231,14 +1231,16 @@ def depth_average(hist: torch.Tensor, count: int, weights: torch.Tensor, last: t
 
 def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: torch.Tensor, q_start: torch.Tensor,
                      slots: torch.Tensor, heads: int, key_dim: int, value_dim: int, decay: torch.Tensor | None = None,
-                     forget_bias: torch.Tensor | None = None, forget_low: torch.Tensor | None = None) -> torch.Tensor:
+                     forget_bias: torch.Tensor | None = None, forget_low: torch.Tensor | None = None,
+                     longest: int | None = None) -> torch.Tensor:
     """The recurrence ``S_t = diag(a_t) S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t`` per head over every request's
     tokens of this step, from the 32-bit sums ``proj`` of one stacked product (columns from ``q_off``, ``k_off``
     and ``v_off`` on, head by head).  With ``decay`` (32-bit, one number a head): q, k and v pass silu and a_t is
     the head's decay.  With ``forget_bias`` and ``forget_low`` (32-bit [heads * key_dim]): q passes silu, the
     columns at ``k_off`` are a forget gate's, f = low + (1 - low) * sigmoid(. + bias), a_t = f and k_t = 1 - f, v as
     it is.  ``state`` [slots + 1, heads * value_dim * key_dim] (32-bit) is read and written in the requests'
-    ``slots``.  Returns o [tokens, heads * value_dim] in 32-bit."""
+    ``slots``.  ``longest``: the most tokens a request brings in this step (the launch's form depends on it, the sums
+    do not; by default the step's tokens).  Returns o [tokens, heads * value_dim] in 32-bit."""
     _gpu(proj, state, q_start, slots, decay, forget_bias, forget_low)
     _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1, "linear_attention: 32-bit rows with unit inner stride")
     H, dk, dv = int(heads), int(key_dim), int(value_dim)
@@ -1263,7 +1265,8 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, sta
         call("tk_linear_attention", 0 if constant else 1, proj.data_ptr(), proj.stride(0), int(q_off), int(k_off), int(v_off),
              decay.data_ptr() if constant else None, forget_bias.data_ptr() if not constant else None,
              forget_low.data_ptr() if not constant else None, state.data_ptr(), state.stride(0), q_start.data_ptr(),
-             slots.data_ptr(), rec.data_ptr(), o.data_ptr(), n, slots.numel(), H, dk, dv, _stream())
+             slots.data_ptr(), rec.data_ptr(), o.data_ptr(), n, slots.numel(), H, dk, dv, int(n if longest is None else longest),
+             _stream())
     return o
 
 

@@ -89,7 +89,7 @@ class LightningAttention(_LinearAttention):
         assert state is not None, "linear attention keeps its state in the request's slot"
         H, dk, dv = self.num_heads, self.key_dim, self.value_dim
         proj = self.inp(h, out_f32=True)
-        o = ops.linear_attention(proj, 0, H * dk, 2 * H * dk, state, ctx.q_start, ctx.slots, H, dk, dv, decay=self.decay)
+        o = ops.linear_attention(proj, 0, H * dk, 2 * H * dk, state, ctx.q_start, ctx.slots, H, dk, dv, decay=self.decay, longest=ctx.max_q_len)
         gate = proj[:, 2 * H * dk + H * dv :]
         return ops.group_norm_gate(o, self.norm_w, self.norm_eps, 1, h.dtype, gate=gate, scale=scale, out=out)
 
@@ -128,5 +128,5 @@ class HGRN2(_LinearAttention):
         H, dk, dv = self.num_heads, self.key_dim, self.value_dim
         proj = self.inp(h, out_f32=True)
         o = ops.linear_attention(proj, 0, H * dk, 2 * H * dk, state, ctx.q_start, ctx.slots, H, dk, dv,
-                                 forget_bias=self.f_bias, forget_low=self.f_low)
+                                 forget_bias=self.f_bias, forget_low=self.f_low, longest=ctx.max_q_len)
         return ops.group_norm_gate(o, self.norm_w, self.norm_eps, H, h.dtype, scale=scale, out=out)
