@@ -46,7 +46,7 @@ def step_arrays(lens, slots):
 
 
 @pytest.mark.parametrize("heads, dk, dv, lens", [(2, 16, 16, [1, 1, 1]), (3, 12, 6, [3, 40, 1, 9]), (1, 128, 64, [70, 7]),
-                                                 (2, 50, 20, [33]), (1, 200, 8, [5, 18])])
+                                                 (2, 50, 20, [33]), (1, 200, 8, [5, 18]), (1, 300, 8, [9, 3]), (1, 512, 4, [6])])
 @pytest.mark.parametrize("form", ["constant", "forget"])
 def test_linear_attention_kernel(heads, dk, dv, lens, form):
     """The recurrence on random sums, from random states in shuffled slots, against the plain loop; then the same

@@ -26,8 +26,8 @@ __device__ __forceinline__ float la_sigmoid(float x) { return 1.0f / (1.0f + exp
 
 // --------------------------------------------------------------------------
 // Before the recurrence, once a token: the activations, into rows that the recurrence's lanes read 16 bytes at a
-// time.  rec row: [q: H x dkp | k or f: H x dkp | v: H x dv (padded to a multiple of 4)], dkp = dk rounded up to a
-// multiple of 64, zeros in the padding (a padded row of S meets a zero of q).
+// time.  rec row: [q: H x dkp | k or f: H x dkp | v: H x dv (padded to a multiple of 4)], dkp = dk rounded up to 64
+// times the pieces a lane holds, zeros in the padding (a padded row of S meets a zero of q).
 //   LA_CONSTANT  q = silu(.), k = silu(.), v = silu(.)
 //   LA_FORGET    q = silu(.), f = low + (1 - low) * sigmoid(. + bias), v as it is
 // --------------------------------------------------------------------------
@@ -153,25 +153,31 @@ __global__ __launch_bounds__(LA_WAVES * TK_WAVE) void linear_attention_kernel(
   }
 }
 
-// Floats of a row of `rec` for these sizes, and the padded size of a head's keys.
+// 16-byte pieces of a head's keys that a lane holds: one of the kernel's instances (1, 2, 3, 4, 6, 8); a head's keys
+// are padded to 64 times that in `rec`.
+static int la_pieces(int dk) {
+  const int nq = (dk + 63) / 64;
+  return nq <= 4 ? nq : (nq <= 6 ? 6 : 8);
+}
+
+// Floats of a row of `rec` for these sizes.
 TK_API int tk_linear_attention_rec_width(int H, int dk, int dv) {
-  const int dkp = (dk + 63) / 64 * 64;
-  return 2 * H * dkp + (H * dv + 3) / 4 * 4;
+  return 2 * H * la_pieces(dk) * 64 + (H * dv + 3) / 4 * 4;
 }
 
 TK_API int tk_linear_attention(int mode, const float* proj, int ld, int q_off, int k_off, int v_off, const float* decay,
                                const float* f_bias, const float* f_low, float* state, size_t state_stride,
                                const int* q_start, const int* slots, float* rec, float* o, int n_tokens, int n_requests, int H,
                                int dk, int dv, int longest, hipStream_t stream) {
-  TK_REQUIRE(n_tokens >= 0 && n_requests >= 0 && H > 0 && dk > 0 && dv > 0 && dk <= 256,
-             "linear_attention: bad sizes tokens=%d requests=%d heads=%d dk=%d dv=%d (dk up to 256)", n_tokens, n_requests, H, dk, dv);
+  TK_REQUIRE(n_tokens >= 0 && n_requests >= 0 && H > 0 && dk > 0 && dv > 0 && dk <= 512,
+             "linear_attention: bad sizes tokens=%d requests=%d heads=%d dk=%d dv=%d (dk up to 512)", n_tokens, n_requests, H, dk, dv);
   TK_REQUIRE(mode == LA_CONSTANT ? decay != nullptr : (mode == LA_FORGET && f_bias && f_low),
              "linear_attention: the constant form needs a decay a head, the forget-gate form a bias and a lower bound");
   TK_REQUIRE(proj && state && q_start && slots && o && rec && state_stride >= (size_t)H * dk * dv && n_requests < 65536 && n_tokens < 65536,
              "linear_attention: a pointer is missing, the state's rows are too short or the step too large");
   TK_REQUIRE((((uintptr_t)rec | (uintptr_t)state) & 15) == 0, "linear_attention: rec and state must start at multiples of 16 bytes");
   if (n_requests == 0 || n_tokens == 0) return 0;
-  const int dkp = (dk + 63) / 64 * 64, nq = dkp / 64;
+  const int nq = la_pieces(dk), dkp = 64 * nq;
   const int ld_rec = tk_linear_attention_rec_width(H, dk, dv);
   const dim3 pgrid((ld_rec + 255) / 256, n_tokens);
   if (mode == LA_CONSTANT)
@@ -197,7 +203,9 @@ TK_API int tk_linear_attention(int mode, const float* proj, int ld, int q_off, i
   if (nq <= 1) LA_CASE(1, 4);
   else if (nq <= 2) LA_CASE(2, 4);
   else if (nq <= 3) LA_CASE(3, 2);
-  else LA_CASE(4, 2);
+  else if (nq <= 4) LA_CASE(4, 2);
+  else if (nq <= 6) LA_CASE(6, 1);
+  else LA_CASE(8, 1);
 #undef LA_CASE
   TK_CHECK_LAUNCH("linear_attention");
   return 0;
@@ -340,6 +348,57 @@ __global__ void short_conv_kernel(const T* __restrict__ h, int ld, const float* 
   out[(size_t)t * width + c] = from_f32<T>(cur + acc);
 }
 
+// The same with 16 bytes a load: a thread 16 / sizeof(T) neighbouring channels (widths and strides that are multiples
+// of that, rows that start at multiples of 16 bytes).
+template <typename T, bool FUSE_TAIL>
+__global__ void short_conv_vec_kernel(const T* __restrict__ h, int ld, const float* __restrict__ w, int taps, float* __restrict__ tails,
+                                      size_t tail_stride, const int* __restrict__ q_start, const int* __restrict__ token_req,
+                                      const int* __restrict__ slots, T* __restrict__ out, int width) {
+  constexpr int N = 16 / sizeof(T);
+  union Piece { uint4 raw; T v[N]; };
+  const int t = blockIdx.y;
+  const int c0 = (blockIdx.x * blockDim.x + threadIdx.x) * N;
+  if (c0 >= width) return;
+  const int r = token_req[t];
+  const int first = q_start[r];
+  const int local = t - first;
+  float* tail = tails + (size_t)slots[r] * tail_stride;
+  float acc[N], cur[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e) acc[e] = cur[e] = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = local - (taps - 1) + j;
+    float x[N];
+    if (src >= 0) {
+      Piece p;
+      p.raw = *(const uint4*)(h + (size_t)(first + src) * ld + c0);
+#pragma unroll
+      for (int e = 0; e < N; ++e) x[e] = to_f32<T>(p.v[e]);
+    } else {
+      const float4* from = (const float4*)(tail + (size_t)(src + taps - 1) * width + c0);
+#pragma unroll
+      for (int e = 0; e < N; e += 4) {
+        const float4 v = from[e / 4];
+        x[e] = v.x; x[e + 1] = v.y; x[e + 2] = v.z; x[e + 3] = v.w;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      acc[e] = fmaf(w[(size_t)(c0 + e) * taps + j], x[e], acc[e]);
+      cur[e] = x[e];
+    }
+    if (FUSE_TAIL && j >= 1) {  // (local is 0: entry j - 1 was read a tap ago)
+      float4* to = (float4*)(tail + (size_t)(j - 1) * width + c0);
+#pragma unroll
+      for (int e = 0; e < N; e += 4) to[e / 4] = make_float4(x[e], x[e + 1], x[e + 2], x[e + 3]);
+    }
+  }
+  Piece o;
+#pragma unroll
+  for (int e = 0; e < N; ++e) o.v[e] = from_f32<T>(cur[e] + acc[e]);
+  *(uint4*)(out + (size_t)t * width + c0) = o.raw;
+}
+
 // The tails after the step: the last taps - 1 inputs of every request, from this step's rows and, where the
 // step brought fewer, from the old tail.  A thread a (request, channel); it reads all it needs before it writes.
 template <typename T>
@@ -374,6 +433,30 @@ TK_API int tk_short_conv(int dt, const void* h, int ld, const float* w, int taps
   if (n_tokens == 0) return 0;
   TK_REQUIRE(n_tokens < 65536, "short_conv: %d tokens are too many for one call", n_tokens);
   const dim3 grid((width + 255) / 256, n_tokens), tail_grid((width + 255) / 256, n_requests);
+  const int per = dt == TK_F32 ? 4 : 8;  // channels of 16 bytes
+  const bool vec = width % per == 0 && ld % per == 0 && (((uintptr_t)h | (uintptr_t)out) & 15) == 0 &&
+                   (taps == 1 || ((((uintptr_t)tails) & 15) == 0 && tail_stride % 4 == 0));
+  const dim3 vgrid((width / per + 127) / 128, n_tokens);
+#define SC_VEC(T)                                                                                                                    \
+  do {                                                                                                                               \
+    if (single_tokens)                                                                                                               \
+      hipLaunchKernelGGL((short_conv_vec_kernel<T, true>), vgrid, dim3(128), 0, stream, (const T*)h, ld, w, taps, tails, tail_stride, \
+                         q_start, token_req, slots, (T*)out, width);                                                                 \
+    else {                                                                                                                           \
+      hipLaunchKernelGGL((short_conv_vec_kernel<T, false>), vgrid, dim3(128), 0, stream, (const T*)h, ld, w, taps, tails,            \
+                         tail_stride, q_start, token_req, slots, (T*)out, width);                                                    \
+      if (taps > 1)                                                                                                                  \
+        hipLaunchKernelGGL(short_conv_tail_kernel<T>, tail_grid, dim3(256), 0, stream, (const T*)h, ld, taps, tails, tail_stride,    \
+                           q_start, slots, width);                                                                                   \
+    }                                                                                                                                \
+  } while (0)
+  if (vec) {
+    if (dt == TK_F32) SC_VEC(float);
+    else SC_VEC(bf16_t);
+    TK_CHECK_LAUNCH("short_conv");
+    return 0;
+  }
+#undef SC_VEC
 #define SC_CASE(T)                                                                                                                   \
   do {                                                                                                                               \
     if (single_tokens)                                                                                                               \

@@ -1257,7 +1257,7 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, sta
     _f32_vector(decay, H, "linear_attention: the decays")
     _f32_vector(forget_bias, H * dk, "linear_attention: the forget gate's bias")
     _f32_vector(forget_low, H * dk, "linear_attention: the forget gate's lower bound")
-    _need(dk <= 256, f"linear_attention: heads of up to 256 key channels, not {dk}")
+    _need(dk <= 512, f"linear_attention: heads of up to 512 key channels, not {dk}")
     o = torch.empty((n, H * dv), dtype=torch.float32, device=proj.device)
     if n:
         # the activated rows that the recurrence reads: one pass over the step's tokens in front of it
