@@ -46,7 +46,8 @@ def step_arrays(lens, slots):
 
 
 @pytest.mark.parametrize("heads, dk, dv, lens", [(2, 16, 16, [1, 1, 1]), (3, 12, 6, [3, 40, 1, 9]), (1, 128, 64, [70, 7]),
-                                                 (2, 50, 20, [33]), (1, 200, 8, [5, 18]), (1, 300, 8, [9, 3]), (1, 512, 4, [6])])
+                                                 (2, 50, 20, [33]), (1, 200, 8, [5, 18]), (1, 300, 8, [9, 3]), (1, 512, 4, [6]),
+                                                 (3, 50, 6, [1, 1]), (1, 300, 8, [1]), (2, 128, 40, [1, 1, 1, 1])])
 @pytest.mark.parametrize("form", ["constant", "forget"])
 def test_linear_attention_kernel(heads, dk, dv, lens, form):
     """The recurrence on random sums, from random states in shuffled slots, against the plain loop; then the same
@@ -84,6 +85,12 @@ def test_linear_attention_kernel(heads, dk, dv, lens, form):
         assert torch.allclose(state[slots[r]].cpu().double().view(H, dv, dk), S.transpose(1, 2), atol=2e-4, rtol=2e-4)
         at += ln
     assert torch.equal(state[len(lens)].cpu(), state0[len(lens)])  # a slot of no request stays as it was
+    if max(lens) == 1:
+        # the form for steps of single tokens (activations in the recurrence's own kernel): the same bits
+        state1 = state0.clone().cuda()
+        o1 = ops.linear_attention(proj.cuda(), 0, H * dk, 2 * H * dk, state1, q_start, slot_t, H, dk, dv, decay=dev(decay),
+                                  forget_bias=dev(bias), forget_low=dev(low), longest=1)
+        assert torch.equal(o1, o) and torch.equal(state1, state)
     # the same tokens in two steps, cut inside every request that has two tokens or more
     cut = [max(1, ln // 3) if ln > 1 else 1 for ln in lens]
     state2 = state0.clone().cuda()

@@ -34,7 +34,7 @@ def test_positions_enter_through_the_embedding():
 
 def test_distance_buckets():
     # every short distance has a bucket of its own; the others climb on a logarithmic scale and end in the last bucket
-    for buckets, far in ((16, 240), (2, 7), (8, 20), (64, 4000), (12, 100)):
+    for buckets, far in ((14, 200), (2, 7), (8, 20), (64, 4000), (12, 100)):
         got = [pz.distance_bucket(n, buckets, far) for n in range(far + 50)]
         half = buckets // 2
         assert got[:half] == list(range(half)) and got[half] == half

@@ -23,6 +23,8 @@ enum { LA_CONSTANT = 0, LA_FORGET = 1 };
 
 __device__ __forceinline__ float la_silu(float x) { return x / (1.0f + expf(-x)); }
 __device__ __forceinline__ float la_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+// the forget gate, written out in one multiply-add so that every kernel that computes it gets the same bits
+__device__ __forceinline__ float la_forget(float x, float bias, float lo) { return fmaf(1.0f - lo, la_sigmoid(x + bias), lo); }
 
 // --------------------------------------------------------------------------
 // Before the recurrence, once a token: the activations, into rows that the recurrence's lanes read 16 bytes at a
@@ -49,8 +51,7 @@ __global__ __launch_bounds__(256) void linear_attention_prepare_kernel(
       } else if (MODE == LA_CONSTANT) {
         val = la_silu(row[k_off + c]);
       } else {
-        const float lo = f_low[c];
-        val = lo + (1.0f - lo) * la_sigmoid(row[k_off + c] + f_bias[c]);
+        val = la_forget(row[k_off + c], f_bias[c], f_low[c]);
       }
     }
   } else {
@@ -160,6 +161,73 @@ static int la_pieces(int dk) {
   return nq <= 4 ? nq : (nq <= 6 ? 6 : 8);
 }
 
+// --------------------------------------------------------------------------
+// The same for steps in which every request brings one token: the activations are computed by the lanes that need
+// them (there is no pass in front and no `rec`), with the functions of the pass above, so the sums are the same bits.
+// --------------------------------------------------------------------------
+template <int NQ, int MODE>
+__global__ __launch_bounds__(LA_WAVES * TK_WAVE) void linear_attention_single_kernel(
+    const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
+    const float* __restrict__ f_bias, const float* __restrict__ f_low, float* __restrict__ state, size_t state_stride,
+    const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ o, int H, int dk, int dv) {
+  const int h = blockIdx.x, r = blockIdx.y;
+  const int lane = threadIdx.x % LA_LANES, grp = threadIdx.x / LA_LANES;
+  const int col = blockIdx.z * (blockDim.x / LA_LANES) + grp;
+  if ((col / LA_COLS) * LA_COLS >= dv) return;
+  const bool live = col < dv;
+  const int t = q_start[r];
+  if (q_start[r + 1] <= t) return;
+  float* s_col = state + (size_t)slots[r] * state_stride + ((size_t)h * dv + (live ? col : 0)) * dk;
+  const bool vec = (dk % 4 == 0) && (state_stride % 4 == 0);
+  const float* row = proj + (size_t)t * ld;
+  const float a_head = MODE == LA_CONSTANT ? decay[h] : 0.f;
+  const float raw_v = row[v_off + h * dv + (live ? col : 0)];
+  const float vv = MODE == LA_CONSTANT ? la_silu(raw_v) : raw_v;
+  float acc0 = 0.f, acc1 = 0.f;
+  float s[NQ][4];
+#pragma unroll
+  for (int n = 0; n < NQ; ++n) {
+    const int i = 4 * (lane + LA_LANES * n);
+    if (vec && live && i < dk) {
+      const float4 v = *(const float4*)(s_col + i);
+      s[n][0] = v.x; s[n][1] = v.y; s[n][2] = v.z; s[n][3] = v.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[n][e] = (live && i + e < dk) ? s_col[i + e] : 0.f;
+    }
+    float qq[4], kk[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool in = i + e < dk;
+      const int c = h * dk + (in ? i + e : 0);
+      qq[e] = in ? la_silu(row[q_off + c]) : 0.f;
+      if (MODE == LA_CONSTANT) kk[e] = in ? la_silu(row[k_off + c]) : 0.f;
+      else kk[e] = in ? la_forget(row[k_off + c], f_bias[c], f_low[c]) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (MODE == LA_CONSTANT) s[n][e] = fmaf(a_head, s[n][e], kk[e] * vv);
+      else s[n][e] = fmaf(kk[e], s[n][e] - vv, vv);
+    }
+    acc0 = fmaf(qq[0], s[n][0], acc0); acc1 = fmaf(qq[1], s[n][1], acc1);
+    acc0 = fmaf(qq[2], s[n][2], acc0); acc1 = fmaf(qq[3], s[n][3], acc1);
+  }
+  const float sum = row_sum16(acc0 + acc1);
+  if (!live) return;
+  if (lane == 0) o[(size_t)t * H * dv + (size_t)h * dv + col] = sum;
+#pragma unroll
+  for (int n = 0; n < NQ; ++n) {
+    const int i = 4 * (lane + LA_LANES * n);
+    if (vec && i < dk) {
+      *(float4*)(s_col + i) = make_float4(s[n][0], s[n][1], s[n][2], s[n][3]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (i + e < dk) s_col[i + e] = s[n][e];
+    }
+  }
+}
+
 // Floats of a row of `rec` for these sizes.
 TK_API int tk_linear_attention_rec_width(int H, int dk, int dv) {
   return 2 * H * la_pieces(dk) * 64 + (H * dv + 3) / 4 * 4;
@@ -173,11 +241,35 @@ TK_API int tk_linear_attention(int mode, const float* proj, int ld, int q_off, i
              "linear_attention: bad sizes tokens=%d requests=%d heads=%d dk=%d dv=%d (dk up to 512)", n_tokens, n_requests, H, dk, dv);
   TK_REQUIRE(mode == LA_CONSTANT ? decay != nullptr : (mode == LA_FORGET && f_bias && f_low),
              "linear_attention: the constant form needs a decay a head, the forget-gate form a bias and a lower bound");
-  TK_REQUIRE(proj && state && q_start && slots && o && rec && state_stride >= (size_t)H * dk * dv && n_requests < 65536 && n_tokens < 65536,
+  const bool single = longest <= 1;
+  TK_REQUIRE(proj && state && q_start && slots && o && (rec || single) && state_stride >= (size_t)H * dk * dv && n_requests < 65536 && n_tokens < 65536,
              "linear_attention: a pointer is missing, the state's rows are too short or the step too large");
   TK_REQUIRE((((uintptr_t)rec | (uintptr_t)state) & 15) == 0, "linear_attention: rec and state must start at multiples of 16 bytes");
+  TK_REQUIRE(longest >= 1, "linear_attention: the longest portion of a step with tokens is at least one token");
   if (n_requests == 0 || n_tokens == 0) return 0;
   const int nq = la_pieces(dk), dkp = 64 * nq;
+  if (single) {
+    const int waves = min(LA_WAVES, (dv + LA_COLS - 1) / LA_COLS);
+    const dim3 grid(H, n_requests, (dv + LA_COLS * waves - 1) / (LA_COLS * waves)), block(waves * TK_WAVE);
+#define LA_SINGLE(NQ)                                                                                                           \
+  do {                                                                                                                          \
+    if (mode == LA_CONSTANT)                                                                                                    \
+      hipLaunchKernelGGL((linear_attention_single_kernel<NQ, LA_CONSTANT>), grid, block, 0, stream, proj, ld, q_off, k_off,     \
+                         v_off, decay, f_bias, f_low, state, state_stride, q_start, slots, o, H, dk, dv);                       \
+    else                                                                                                                        \
+      hipLaunchKernelGGL((linear_attention_single_kernel<NQ, LA_FORGET>), grid, block, 0, stream, proj, ld, q_off, k_off, v_off, \
+                         decay, f_bias, f_low, state, state_stride, q_start, slots, o, H, dk, dv);                              \
+  } while (0)
+    if (nq <= 1) LA_SINGLE(1);
+    else if (nq <= 2) LA_SINGLE(2);
+    else if (nq <= 3) LA_SINGLE(3);
+    else if (nq <= 4) LA_SINGLE(4);
+    else if (nq <= 6) LA_SINGLE(6);
+    else LA_SINGLE(8);
+#undef LA_SINGLE
+    TK_CHECK_LAUNCH("linear_attention");
+    return 0;
+  }
   const int ld_rec = tk_linear_attention_rec_width(H, dk, dv);
   const dim3 pgrid((ld_rec + 255) / 256, n_tokens);
   if (mode == LA_CONSTANT)

@@ -1260,12 +1260,15 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, sta
     _need(dk <= 512, f"linear_attention: heads of up to 512 key channels, not {dk}")
     o = torch.empty((n, H * dv), dtype=torch.float32, device=proj.device)
     if n:
-        # the activated rows that the recurrence reads: one pass over the step's tokens in front of it
-        rec = torch.empty((n, load("core").tk_linear_attention_rec_width(H, dk, dv)), dtype=torch.float32, device=proj.device)
+        longest = int(n if longest is None else longest)
+        # the activated rows that the recurrence reads: one pass over the step's tokens in front of it (a step of single
+        # tokens computes them in the recurrence's own kernel)
+        rec = (torch.empty((n, load("core").tk_linear_attention_rec_width(H, dk, dv)), dtype=torch.float32, device=proj.device)
+               if longest > 1 else None)
         call("tk_linear_attention", 0 if constant else 1, proj.data_ptr(), proj.stride(0), int(q_off), int(k_off), int(v_off),
              decay.data_ptr() if constant else None, forget_bias.data_ptr() if not constant else None,
              forget_low.data_ptr() if not constant else None, state.data_ptr(), state.stride(0), q_start.data_ptr(),
-             slots.data_ptr(), rec.data_ptr(), o.data_ptr(), n, slots.numel(), H, dk, dv, int(n if longest is None else longest),
+             slots.data_ptr(), rec.data_ptr() if rec is not None else None, o.data_ptr(), n, slots.numel(), H, dk, dv, longest,
              _stream())
     return o
 
