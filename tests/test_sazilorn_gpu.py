@@ -133,7 +133,7 @@ def test_short_convolution_kernel(dtype, width, taps, lens):
     for half in (0, 1):
         rows = torch.cat([s[half * ln : (half + 1) * ln] for s, ln in zip(seqs, lens)]).cuda()
         q_start, req, slot_t = step_arrays(lens, slots)
-        out = ops.short_conv(rows, w.cuda(), tails if taps > 1 else None, q_start, req, slot_t, single_tokens=max(lens) == 1)
+        out = ops.short_conv(rows, w.t().contiguous().cuda(), tails if taps > 1 else None, q_start, req, slot_t, single_tokens=max(lens) == 1)
         at = 0
         for r, ln in enumerate(lens):
             ref = want[r][half * ln : (half + 1) * ln]

@@ -411,7 +411,8 @@ TK_API int tk_sigmoid_gate(int dt, const void* x, int ld_x, const void* gate, in
 
 // --------------------------------------------------------------------------
 // A short causal convolution over time on every channel, added to its input:
-//     out_t = h_t + sum_j w[c][j] * h_(t - taps + 1 + j)      (zeros before a request's first token)
+//     out_t = h_t + sum_j w[j][c] * h_(t - taps + 1 + j)      (zeros before a request's first token)
+// The taps are kept tap by tap, w [taps][width], so that neighbouring channels' weights of one tap lie together.
 // The last taps - 1 inputs of a request live in its slot's `tail` [taps - 1][width] (32-bit, oldest first,
 // zeros when the request takes the slot).  A thread a (token, channel).  FUSE_TAIL (every request of the step
 // brings one token): the thread also moves its channel's tail on, which it alone reads; else the tail kernel
@@ -433,7 +434,7 @@ __global__ void short_conv_kernel(const T* __restrict__ h, int ld, const float* 
   for (int j = 0; j < taps; ++j) {
     const int src = local - (taps - 1) + j;
     const float x = src >= 0 ? to_f32<T>(h[(size_t)(first + src) * ld + c]) : tail[(size_t)(src + taps - 1) * width + c];
-    acc = fmaf(w[(size_t)c * taps + j], x, acc);
+    acc = fmaf(w[(size_t)j * width + c], x, acc);
     cur = x;
     if (FUSE_TAIL && j >= 1) tail[(size_t)(j - 1) * width + c] = x;  // (local is 0: entry j - 1 was read a tap ago)
   }
@@ -458,6 +459,7 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ h, int ld, const flo
   float acc[N], cur[N];
 #pragma unroll
   for (int e = 0; e < N; ++e) acc[e] = cur[e] = 0.f;
+#pragma unroll 4
   for (int j = 0; j < taps; ++j) {
     const int src = local - (taps - 1) + j;
     float x[N];
@@ -474,11 +476,15 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ h, int ld, const flo
         x[e] = v.x; x[e + 1] = v.y; x[e + 2] = v.z; x[e + 3] = v.w;
       }
     }
+    const float4* wj = (const float4*)(w + (size_t)j * width + c0);
 #pragma unroll
-    for (int e = 0; e < N; ++e) {
-      acc[e] = fmaf(w[(size_t)(c0 + e) * taps + j], x[e], acc[e]);
-      cur[e] = x[e];
+    for (int e = 0; e < N; e += 4) {
+      const float4 g = wj[e / 4];
+      acc[e] = fmaf(g.x, x[e], acc[e]); acc[e + 1] = fmaf(g.y, x[e + 1], acc[e + 1]);
+      acc[e + 2] = fmaf(g.z, x[e + 2], acc[e + 2]); acc[e + 3] = fmaf(g.w, x[e + 3], acc[e + 3]);
     }
+#pragma unroll
+    for (int e = 0; e < N; ++e) cur[e] = x[e];
     if (FUSE_TAIL && j >= 1) {  // (local is 0: entry j - 1 was read a tap ago)
       float4* to = (float4*)(tail + (size_t)(j - 1) * width + c0);
 #pragma unroll
@@ -526,7 +532,7 @@ TK_API int tk_short_conv(int dt, const void* h, int ld, const float* w, int taps
   TK_REQUIRE(n_tokens < 65536, "short_conv: %d tokens are too many for one call", n_tokens);
   const dim3 grid((width + 255) / 256, n_tokens), tail_grid((width + 255) / 256, n_requests);
   const int per = dt == TK_F32 ? 4 : 8;  // channels of 16 bytes
-  const bool vec = width % per == 0 && ld % per == 0 && (((uintptr_t)h | (uintptr_t)out) & 15) == 0 &&
+  const bool vec = width % per == 0 && ld % per == 0 && (((uintptr_t)h | (uintptr_t)out | (uintptr_t)w) & 15) == 0 &&
                    (taps == 1 || ((((uintptr_t)tails) & 15) == 0 && tail_stride % 4 == 0));
   const dim3 vgrid((width / per + 127) / 128, n_tokens);
 #define SC_VEC(T)                                                                                                                    \

@@ -1317,16 +1317,17 @@ def sigmoid_gate(x: torch.Tensor, gate: torch.Tensor, scale: float = 1.0, out: t
 
 def short_conv(h: torch.Tensor, weight: torch.Tensor, tails: torch.Tensor | None, q_start: torch.Tensor, token_req: torch.Tensor,
                slots: torch.Tensor, single_tokens: bool) -> torch.Tensor:
-    """h + conv(h) with a causal convolution over time on every channel, ``conv(h)_t = sum_j weight[:, j] *
-    h_(t - taps + 1 + j)``, zeros before a request's start.  ``weight`` [width, taps] in 32-bit; ``tails``
+    """h + conv(h) with a causal convolution over time on every channel, ``conv(h)_t = sum_j weight[j] *
+    h_(t - taps + 1 + j)``, zeros before a request's start.  ``weight`` [taps, width] in 32-bit (tap by tap; the last
+    row is the current token's); ``tails``
     [slots + 1, (taps - 1) * width] (32-bit) holds every request's last taps - 1 inputs and is moved on.
     ``single_tokens``: every request of the step brings one token (the tails then move in the same kernel)."""
     _gpu(h, weight, tails, q_start, token_req, slots)
     _need(h.dim() == 2 and h.stride(1) == 1, "short_conv: rows with unit inner stride")
     n, width = h.shape
-    _need(weight.dim() == 2 and weight.shape[0] == width and weight.dtype == torch.float32 and weight.is_contiguous(),
-          "short_conv: taps must be contiguous float32 [width, taps]")
-    taps = weight.shape[1]
+    _need(weight.dim() == 2 and weight.shape[1] == width and weight.dtype == torch.float32 and weight.is_contiguous(),
+          "short_conv: taps must be contiguous float32 [taps, width]")
+    taps = weight.shape[0]
     if taps > 1:
         _need(tails is not None and tails.dim() == 2 and tails.dtype == torch.float32 and tails.is_contiguous()
               and tails.shape[1] >= (taps - 1) * width, "short_conv: the tails must be contiguous float32 [slots, (taps - 1) * width]")

@@ -30,7 +30,8 @@ class ShortConvResidual(Part):
         return StateNeed(((self.taps - 1) * self.width,), torch.float32) if self.taps > 1 else None
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
-        self.weight = placer.place(("conv_f32", self.name), lambda: tensors[self.name].to(torch.float32).contiguous().to(placer.device))
+        # tap by tap, [taps, width]: neighbouring channels' weights of one tap lie together
+        self.weight = placer.place(("conv_f32_by_tap", self.name), lambda: tensors[self.name].to(torch.float32).t().contiguous().to(placer.device))
 
     def forward(self, h: torch.Tensor, ctx: StepContext, tails: torch.Tensor | None) -> torch.Tensor:
         if self.taps > 1 and tails is None:
