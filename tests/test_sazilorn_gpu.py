@@ -196,6 +196,38 @@ def test_gelu_gate_and_sigmoid_gate_kernels():
     assert float(out[:, :40].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("groups, size", [(1, 1024), (1, 300), (3, 20), (2, 512), (1, 4100)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_behind_the_recurrence(groups, size, dtype):
+    """Every group's numbers over their root mean square, times the shared weight, the gate's sigmoid and a factor,
+    into columns of a wider buffer: a wavefront a group for small groups, a workgroup for large ones."""
+    torch.manual_seed(size)
+    n = 5
+    o, w = torch.randn(n, groups * size), torch.randn(size)
+    gate = torch.randn(n, groups * size + 8)
+    out = torch.zeros(n, groups * size + 16, dtype=dtype).cuda()
+    for g in (None, gate):
+        view = out[:, 16:]
+        ops.group_norm_gate(o.cuda(), w.cuda(), 1e-5, groups, dtype, gate=None if g is None else g.cuda()[:, 8:], scale=0.7, out=view)
+        want = pz.rms(o.double().view(n, groups, size), 1e-5) * w.double()
+        if g is not None:
+            want = want * torch.sigmoid(g[:, 8:].double().view(n, groups, size))
+        tol = 1e-5 if dtype == torch.float32 else 2e-2
+        assert torch.allclose(view.cpu().double(), want.reshape(n, -1) * 0.7, atol=tol, rtol=tol)
+    assert float(out[:, :16].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gate_per_element_with_16_byte_loads(dtype):
+    torch.manual_seed(6)
+    x, g = torch.randn(6, 128).to(dtype), torch.randn(6, 256 + 64).to(dtype)
+    out = torch.zeros(6, 128 + 64, dtype=dtype).cuda()
+    ops.sigmoid_gate(x.cuda(), g.cuda()[:, 64:192], scale=1.5, out=out[:, :128])
+    want = x.double() * torch.sigmoid(g[:, 64:192].double()) * 1.5
+    tol = 1e-6 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(out[:, :128].cpu().double(), want, atol=tol, rtol=tol) and float(out[:, 128:].abs().max()) == 0.0
+
+
 # ---------------------------------------------------------------------------------- one mechanism a model
 
 

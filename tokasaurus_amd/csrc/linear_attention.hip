@@ -341,6 +341,33 @@ __global__ __launch_bounds__(256) void group_norm_gate_wide_kernel(const float* 
   const int g = (int)(unit % groups);
   const float* x = o + (size_t)unit * size;
   float ss = 0.f;
+  if (size % 4 == 0 && size <= 4 * 256 * 4 && ((uintptr_t)x & 15) == 0) {
+    // the row in registers: up to four 16-byte pieces a thread, asked for together
+    float4 v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i = threadIdx.x + q * 256;
+      v[q] = i < size / 4 ? ((const float4*)x)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      ss = fmaf(v[q].x, v[q].x, ss); ss = fmaf(v[q].y, v[q].y, ss); ss = fmaf(v[q].z, v[q].z, ss); ss = fmaf(v[q].w, v[q].w, ss);
+    }
+    ss = block_sum(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)size + eps);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i = threadIdx.x + q * 256;
+      if (i < size / 4) {
+        const float xs[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int c = 4 * i + e;
+          float y = xs[e] * rstd * w[c];
+          if (gate) y *= la_sigmoid(gate[(size_t)t * ld_gate + (size_t)g * size + c]);
+          out[(size_t)t * ld_out + (size_t)g * size + c] = from_f32<T>(y * scale);
+        }
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < size; i += blockDim.x) ss = fmaf(x[i], x[i], ss);
   ss = block_sum(ss, red);
   const float rstd = 1.0f / sqrtf(ss / (float)size + eps);
@@ -393,12 +420,42 @@ __global__ void sigmoid_gate_kernel(const T* __restrict__ x, int ld_x, const T* 
     out[t * ld_out + i] = from_f32<T>(to_f32<T>(x[t * ld_x + i]) * la_sigmoid(to_f32<T>(gate[t * ld_gate + i])) * scale);
 }
 
+// (16 bytes a load where widths, strides and addresses allow)
+template <typename T>
+__global__ void sigmoid_gate_vec_kernel(const T* __restrict__ x, int ld_x, const T* __restrict__ gate, int ld_gate, float scale,
+                                        T* __restrict__ out, int ld_out, int width) {
+  constexpr int N = 16 / sizeof(T);
+  union Piece { uint4 raw; T v[N]; };
+  const int i = (blockIdx.x * blockDim.x + threadIdx.x) * N;
+  const size_t t = blockIdx.y;
+  if (i >= width) return;
+  Piece a, g, o;
+  a.raw = *(const uint4*)(x + t * ld_x + i);
+  g.raw = *(const uint4*)(gate + t * ld_gate + i);
+#pragma unroll
+  for (int e = 0; e < N; ++e) o.v[e] = from_f32<T>(to_f32<T>(a.v[e]) * la_sigmoid(to_f32<T>(g.v[e])) * scale);
+  *(uint4*)(out + t * ld_out + i) = o.raw;
+}
+
 TK_API int tk_sigmoid_gate(int dt, const void* x, int ld_x, const void* gate, int ld_gate, float scale, void* out, int ld_out,
                            int rows, int width, hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && rows < 65536 && width > 0 && x && gate && out && ld_x >= width && ld_gate >= width && ld_out >= width,
              "sigmoid_gate: bad sizes %d %d, a pointer is missing or a stride is too short", rows, width);
   if (rows == 0) return 0;
   const dim3 grid((width + 255) / 256, rows);
+  const int per = dt == TK_F32 ? 4 : 8;
+  if (width % per == 0 && ld_x % per == 0 && ld_gate % per == 0 && ld_out % per == 0 &&
+      (((uintptr_t)x | (uintptr_t)gate | (uintptr_t)out) & 15) == 0) {
+    const dim3 vgrid((width / per + 127) / 128, rows);
+    if (dt == TK_F32)
+      hipLaunchKernelGGL(sigmoid_gate_vec_kernel<float>, vgrid, dim3(128), 0, stream, (const float*)x, ld_x, (const float*)gate,
+                         ld_gate, scale, (float*)out, ld_out, width);
+    else
+      hipLaunchKernelGGL(sigmoid_gate_vec_kernel<bf16_t>, vgrid, dim3(128), 0, stream, (const bf16_t*)x, ld_x, (const bf16_t*)gate,
+                         ld_gate, scale, (bf16_t*)out, ld_out, width);
+    TK_CHECK_LAUNCH("sigmoid_gate");
+    return 0;
+  }
   if (dt == TK_F32)
     hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, ld_x, (const float*)gate, ld_gate,
                        scale, (float*)out, ld_out, width);
