@@ -1260,7 +1260,7 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, sta
     _need(dk <= 512, f"linear_attention: heads of up to 512 key channels, not {dk}")
     o = torch.empty((n, H * dv), dtype=torch.float32, device=proj.device)
     if n:
-        longest = int(n if longest is None else longest)
+        longest = max(1, int(n if longest is None else longest))
         # the activated rows that the recurrence reads: one pass over the step's tokens in front of it (a step of single
         # tokens computes them in the recurrence's own kernel)
         rec = (torch.empty((n, load("core").tk_linear_attention_rec_width(H, dk, dv)), dtype=torch.float32, device=proj.device)
